@@ -1,0 +1,229 @@
+"""Python host side of the MI355X GEMM hot path: a ctypes binding of lib/libckopt.so.
+
+The functions mirror the reference's host launchers (same names, parameter order and meaning;
+matmul_shmem.cu:143-152, matmul_shmem_tc_async_opt_port_{0,1,2}.cu launchers) and raise CkoptError
+where the reference asserts. They take raw device pointers (ints), so any allocator works; torch
+tensors are accepted for convenience and only their data_ptr() is used.
+
+The directory name contains a hyphen, so load it with importlib (see __graft_entry__.load_package()).
+There is no CPU fallback: if the HIP library is missing, importing this module fails.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libckopt.so")
+
+DT_F16, DT_BF16, DT_F32, DT_I32 = 0, 1, 2, 3
+OK, ERR_BAD_PARAM, ERR_LDS_BUDGET, ERR_NO_INSTANCE, ERR_HIP, ERR_ALIGNMENT, ERR_NULL, ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6, -7
+OPT_SWIZZLE, OPT_SPIN_LIMIT, OPT_NUM_XCD = 0, 1, 2
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "libckopt.so is not built (%s); run `python cuda-kernel-opt_amd/build.py` - there is no CPU fallback" % LIB_PATH)
+
+_lib = ctypes.CDLL(LIB_PATH)
+_i, _f, _p, _i64, _u64 = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64
+
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
+_lib.ckopt_gemm_shmem_tc_async_opt_port_1.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_1.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 12 + [_p]
+_lib.ckopt_gemm_shmem_tc_async_opt_port_0.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_0.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 10 + [_p]
+_lib.ckopt_get_lds_req.restype = _i
+_lib.ckopt_get_lds_req.argtypes = [_i] * 8
+_lib.ckopt_get_num_acc.restype = _i
+_lib.ckopt_get_num_acc.argtypes = [_i, _i]
+_lib.ckopt_get_warp_tile_rows.restype = _i
+_lib.ckopt_get_warp_tile_rows.argtypes = [_i, _i]
+_lib.ckopt_get_tile_offset_cd.restype = _i64
+_lib.ckopt_get_tile_offset_cd.argtypes = [_i, _i, _i, _i, _i64]
+_lib.ckopt_check_gemm_tuning.restype = _i
+_lib.ckopt_check_gemm_tuning.argtypes = [_i] * 11
+_lib.ckopt_matmul_shmem.restype = _i
+_lib.ckopt_matmul_shmem.argtypes = [_i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]
+_lib.ckopt_matmul_shmem_lds_req.restype = _i
+_lib.ckopt_matmul_shmem_lds_req.argtypes = [_i, _i]
+_lib.ckopt_check_matmul_shmem_tuning.restype = _i
+_lib.ckopt_check_matmul_shmem_tuning.argtypes = [_i, _i]
+_lib.ckopt_device_status.restype = _i
+_lib.ckopt_device_status.argtypes = [_p]
+_lib.ckopt_set_option.restype = _i
+_lib.ckopt_set_option.argtypes = [_i, _i]
+_lib.ckopt_fill_uniform.restype = _i
+_lib.ckopt_fill_uniform.argtypes = [_i, _p, _i64, _u64, _u64, _f, _f]
+_lib.ckopt_fill_normal.restype = _i
+_lib.ckopt_fill_normal.argtypes = [_i, _p, _i64, _u64, _u64, _f, _f]
+_lib.ckopt_fill_int.restype = _i
+_lib.ckopt_fill_int.argtypes = [_i, _p, _i64, _u64, _u64, _i, _i]
+_lib.ckopt_fill_constant.restype = _i
+_lib.ckopt_fill_constant.argtypes = [_i, _p, _i64, _f]
+_lib.ckopt_error_string.restype = ctypes.c_char_p
+_lib.ckopt_error_string.argtypes = [_i]
+
+EXPORTED_SYMBOLS = [
+    "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_1",
+    "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
+    "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
+    "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_set_option", "ckopt_fill_uniform",
+    "ckopt_fill_normal", "ckopt_fill_int", "ckopt_fill_constant", "ckopt_error_string",
+]
+
+
+class CkoptError(RuntimeError):
+    def __init__(self, code, where):
+        self.code = code
+        super().__init__("%s: %s (%d)" % (where, error_string(code), code))
+
+
+def error_string(code):
+    return _lib.ckopt_error_string(code).decode()
+
+
+def _check(code, where):
+    if code != OK:
+        raise CkoptError(code, where)
+
+
+def _dptr(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return ctypes.c_void_p(x)
+    return ctypes.c_void_p(x.data_ptr())  # torch tensor
+
+
+def _stream(stream):
+    if stream is None:
+        return None
+    if isinstance(stream, int):
+        return ctypes.c_void_p(stream)
+    return ctypes.c_void_p(stream.cuda_stream)  # torch.cuda.Stream
+
+
+def get_num_acc(tile_dim, num_consumer_waves):
+    r = _lib.ckopt_get_num_acc(tile_dim, num_consumer_waves)
+    if r < 0:
+        raise CkoptError(r, "get_num_acc")
+    return r
+
+
+def get_warp_tile_rows(tile_dim, num_consumer_waves):
+    r = _lib.ckopt_get_warp_tile_rows(tile_dim, num_consumer_waves)
+    if r < 0:
+        raise CkoptError(r, "get_warp_tile_rows")
+    return r
+
+
+def get_tile_offset_cd(M, N, tile_dim, tile_group_m, tile_count):
+    r = _lib.ckopt_get_tile_offset_cd(M, N, tile_dim, tile_group_m, tile_count)
+    if r < 0:
+        raise CkoptError(int(r), "get_tile_offset_cd")
+    return int(r)
+
+
+def get_lds_req(tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, num_stages,
+                num_consumer_waves):
+    """Role of the reference's get_shmem_req (port_2.cu:1057-1066)."""
+    r = _lib.ckopt_get_lds_req(tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                               num_stages, num_consumer_waves)
+    if r < 0:
+        raise CkoptError(r, "get_lds_req")
+    return r
+
+
+def check_gemm_tuning(tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m,
+                      num_stages, num_producer_waves, num_consumer_waves, num_cus):
+    return _lib.ckopt_check_gemm_tuning(tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
+                                        bar_step_rows_b, tile_group_m, num_stages, num_producer_waves,
+                                        num_consumer_waves, num_cus)
+
+
+def gemm_shmem_tc_async_opt_port(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+                                 bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages,
+                                 num_producer_warps, num_consumer_warps, num_sms, stream=None):
+    """port_2 launcher (matmul_shmem_tc_async_opt_port_2.cu:1088-1109). B is passed transposed (N x K)."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_2(
+        dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+        bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+        num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port")
+
+
+def gemm_shmem_tc_async_opt_port_1(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_step_rows_a,
+                                   bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps,
+                                   num_sms, stream=None):
+    """port_1 launcher (matmul_shmem_tc_async_opt_port_1.cu:889-908)."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_1(
+        dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_step_rows_a,
+        bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, _stream(stream)),
+        "gemm_shmem_tc_async_opt_port_1")
+
+
+def gemm_shmem_tc_async_opt_port_0(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, tile_group_m,
+                                   num_stages, num_producer_warps, num_consumer_warps, num_sms, stream=None):
+    """port_0 launcher (matmul_shmem_tc_async_opt_port_0.cu:515-532)."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_0(
+        dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, tile_group_m,
+        num_stages, num_producer_warps, num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port_0")
+
+
+def matmul_shmem(dtype, A, B, C, M, N, K, tile_dim, block_rows, b_transposed=False, stream=None):
+    """matmul_shmem launcher (matmul_shmem.cu:143-152); b_transposed selects an N x K B."""
+    _check(_lib.ckopt_matmul_shmem(dtype, _dptr(A), _dptr(B), _dptr(C), M, N, K, tile_dim, block_rows,
+                                   int(b_transposed), _stream(stream)), "matmul_shmem")
+
+
+def matmul_shmem_lds_req(dtype, tile_dim):
+    r = _lib.ckopt_matmul_shmem_lds_req(dtype, tile_dim)
+    if r < 0:
+        raise CkoptError(r, "matmul_shmem_lds_req")
+    return r
+
+
+def check_matmul_shmem_tuning(tile_dim, block_rows):
+    return _lib.ckopt_check_matmul_shmem_tuning(tile_dim, block_rows)
+
+
+def device_status(stream=None):
+    """Synchronises `stream` and returns (and clears) the device status word; raises on HIP errors."""
+    r = _lib.ckopt_device_status(_stream(stream))
+    if r < 0:
+        raise CkoptError(r, "device_status")
+    return r
+
+
+def set_option(key, value):
+    r = _lib.ckopt_set_option(key, value)
+    if r < 0:
+        raise CkoptError(r, "set_option")
+    return r
+
+
+# ---- seeded host inputs (numpy arrays; 16-bit types are returned as float16 / uint16 bit patterns) ----
+def _np_dtype(dtype):
+    import numpy as np
+    return {DT_F16: np.float16, DT_BF16: np.uint16, DT_F32: np.float32, DT_I32: np.int32}[dtype]
+
+
+def _fill(fn, dtype, shape, *args):
+    import numpy as np
+    out = np.empty(shape, dtype=_np_dtype(dtype))
+    _check(fn(dtype, out.ctypes.data_as(ctypes.c_void_p), out.size, *args), fn.__name__)
+    return out
+
+
+def fill_uniform(dtype, shape, seed, stream_id, lo=-1.0, hi=1.0):
+    return _fill(_lib.ckopt_fill_uniform, dtype, shape, seed, stream_id, lo, hi)
+
+
+def fill_normal(dtype, shape, seed, stream_id, mean=0.0, stddev=1.0):
+    return _fill(_lib.ckopt_fill_normal, dtype, shape, seed, stream_id, mean, stddev)
+
+
+def fill_int(dtype, shape, seed, stream_id, lo, hi_inclusive):
+    return _fill(_lib.ckopt_fill_int, dtype, shape, seed, stream_id, lo, hi_inclusive)
+
+
+def fill_constant(dtype, shape, value):
+    return _fill(_lib.ckopt_fill_constant, dtype, shape, value)

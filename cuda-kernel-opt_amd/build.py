@@ -1,0 +1,83 @@
+"""Builds libckopt.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+Usage: python build.py [--jobs N] [--force]
+Every translation unit is compiled to build/<name>.o (in parallel) and linked into lib/libckopt.so
+next to this file. hipcc cross-compiles gfx950 code objects without a GPU.
+"""
+import argparse
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+BUILD = os.path.join(HERE, "build")
+LIBDIR = os.path.join(HERE, "lib")
+LIB = os.path.join(LIBDIR, "libckopt.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+DEVICE_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # packed fp32 VALU forms are kept out of all device code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-x", "c++"]
+
+
+def sources():
+    out = []
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith(".hip") or name.endswith(".cpp"):
+            out.append(os.path.join(CSRC, name))
+    return out
+
+
+def headers_mtime():
+    m = 0.0
+    for root in (CSRC, os.path.join(HERE, "..", "include")):
+        for name in os.listdir(root):
+            if name.endswith((".h", ".inc")):
+                m = max(m, os.path.getmtime(os.path.join(root, name)))
+    return m
+
+
+def compile_one(src, force):
+    obj = os.path.join(BUILD, os.path.basename(src) + ".o")
+    if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), headers_mtime()):
+        return obj, "up to date"
+    flags = DEVICE_FLAGS if src.endswith(".hip") else HOST_FLAGS
+    cmd = [HIPCC] + flags + ["-c", src, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("compile failed: %s\n%s\n%s" % (" ".join(cmd), r.stdout, r.stderr))
+    return obj, "compiled"
+
+
+def build(jobs=8, force=False, verbose=True):
+    os.makedirs(BUILD, exist_ok=True)
+    os.makedirs(LIBDIR, exist_ok=True)
+    srcs = sources()
+    objs = []
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        for obj, what in ex.map(lambda s: compile_one(s, force), srcs):
+            if verbose:
+                print("[build] %-40s %s" % (os.path.basename(obj), what), flush=True)
+            objs.append(obj)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed: %s\n%s\n%s" % (" ".join(cmd), r.stdout, r.stderr))
+    if verbose:
+        print("[build] linked %s" % LIB, flush=True)
+    return LIB
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
+    ap.add_argument("--force", action="store_true")
+    a = ap.parse_args()
+    build(a.jobs, a.force)
+    sys.exit(0)

@@ -1,0 +1,247 @@
+// extern "C" launch layer: parameter validation, instance dispatch, device status word.
+// Declarations and the reference launcher each entry point replaces are in include/ckopt.h.
+#include <hip/hip_runtime.h>
+#include <atomic>
+#include <mutex>
+
+#include "../../include/ckopt.h"
+#include "ck_common.h"
+#include "gemm_pc_kernel.hip.h"
+#include "simt_kernel.hip.h"
+
+namespace ck {
+#define CK_DECL_GEMM(NAME) \
+    hipError_t NAME(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
+CK_DECL_GEMM(launch_gemm_pc_f16_m0) CK_DECL_GEMM(launch_gemm_pc_f16_m1) CK_DECL_GEMM(launch_gemm_pc_f16_m2)
+CK_DECL_GEMM(launch_gemm_pc_bf16_m0) CK_DECL_GEMM(launch_gemm_pc_bf16_m1) CK_DECL_GEMM(launch_gemm_pc_bf16_m2)
+#undef CK_DECL_GEMM
+hipError_t launch_matmul_shmem(int dtype, int tile, int accs, bool bt, dim3 grid, hipStream_t s, const SimtArgs& a);
+}  // namespace ck
+
+// One status word per device; the kernels OR a bit into it when a bounded flag wait gives up.
+__device__ unsigned int ck_status_word = 0;
+
+namespace {
+
+std::atomic<int> g_swizzle{1};
+std::atomic<int> g_spin_limit{1 << 22};
+std::atomic<int> g_num_xcd{8};
+
+constexpr int MAX_DEV = 64;
+std::mutex g_status_mutex;
+unsigned int* g_status_ptr[MAX_DEV] = {};
+
+int status_ptr_for_current_device(unsigned int** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return ck::CK_ERR_HIP;
+    if (dev < 0 || dev >= MAX_DEV) return ck::CK_ERR_HIP;
+    std::lock_guard<std::mutex> lock(g_status_mutex);
+    if (!g_status_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(ck_status_word)) != hipSuccess || !p) return ck::CK_ERR_HIP;
+        g_status_ptr[dev] = static_cast<unsigned int*>(p);
+    }
+    *out = g_status_ptr[dev];
+    return ck::CK_OK;
+}
+
+int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta, int M,
+                int N, int K, const ck::GemmTuning& t, void* stream) {
+    using namespace ck;
+    if (!(dtype == CK_DT_F16 || dtype == CK_DT_BF16)) return CK_ERR_BAD_PARAM;
+    if (M <= 0 || N <= 0 || K <= 0) return CK_ERR_BAD_PARAM;
+    const int rc = check_gemm_tuning(t);
+    if (rc != CK_OK) return rc;
+    if (!A || !Bt || !D) return CK_ERR_NULL;
+    if (beta != 0.f && !C) return CK_ERR_NULL;
+    if (K % CHUNK_ELEMS != 0) return CK_ERR_ALIGNMENT;  // rows must start on 16-byte boundaries
+    if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) return CK_ERR_ALIGNMENT;
+    if (((uintptr_t)D & 3) || ((uintptr_t)C & 3)) return CK_ERR_ALIGNMENT;
+    // one tile's rows are addressed through a 32-bit buffer offset
+    if ((int64_t)t.tile_dim * K * 2 >= (int64_t)1 << 31) return CK_ERR_TOO_LARGE;
+
+    const int mode = sync_mode_of(t.tile_dim, t.num_consumer_waves, t.bar_step_rows_a, t.bar_step_rows_b);
+    GemmArgs a{};
+    a.A = A; a.Bt = Bt; a.C = C; a.D = D;
+    a.alpha = alpha; a.beta = beta;
+    a.M = M; a.N = N; a.K = K;
+    a.tiles_m = (M + t.tile_dim - 1) / t.tile_dim;
+    a.tiles_n = (N + t.tile_dim - 1) / t.tile_dim;
+    a.nseg = (K + t.segment_dim_k - 1) / t.segment_dim_k;
+    a.tile_group_m = t.tile_group_m;
+    a.num_stages = t.num_stages;
+    a.pa = t.num_producer_waves / 2;
+    a.pb = t.num_producer_waves - a.pa;
+    a.bar_steps_a = mode == CK_SYNC_TILE ? 0 : t.bar_steps_a;
+    a.bar_steps_b = mode == CK_SYNC_TILE ? 0 : t.bar_steps_b;
+    a.swizzle = g_swizzle.load();
+    a.num_xcd = g_num_xcd.load();
+    a.vec_store = (N % 4 == 0) && !((uintptr_t)D & 15) && (beta == 0.f || !((uintptr_t)C & 15));
+    a.spin_limit = (uint32_t)g_spin_limit.load();
+    const int src = status_ptr_for_current_device(&a.status);
+    if (src != CK_OK) return src;
+
+    const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+    const int grid = (int)(tiles < t.num_cus ? tiles : t.num_cus);
+    const dim3 block((t.num_producer_waves + t.num_consumer_waves) * WAVE);
+    const size_t lds = (size_t)get_lds_req(t.tile_dim, t.segment_dim_k, a.bar_steps_a, a.bar_steps_b, t.bar_step_rows_a,
+                                           t.bar_step_rows_b, t.num_stages, t.num_consumer_waves);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = hipErrorInvalidValue;
+    if (dtype == CK_DT_F16) {
+        if (mode == 0) e = launch_gemm_pc_f16_m0(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
+        if (mode == 1) e = launch_gemm_pc_f16_m1(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
+        if (mode == 2) e = launch_gemm_pc_f16_m2(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
+    } else {
+        if (mode == 0) e = launch_gemm_pc_bf16_m0(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
+        if (mode == 1) e = launch_gemm_pc_bf16_m1(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
+        if (mode == 2) e = launch_gemm_pc_bf16_m2(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
+    }
+    if (e == hipErrorInvalidValue) return CK_ERR_NO_INSTANCE;
+    return e == hipSuccess ? CK_OK : CK_ERR_HIP;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                         float alpha, float beta, int M, int N, int K, int tile_dim,
+                                         int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                                         int bar_step_rows_b, int tile_group_m, int num_stages,
+                                         int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream);
+}
+
+int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                         float alpha, float beta, int M, int N, int K, int tile_dim,
+                                         int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
+                                         int tile_group_m, int num_stages, int num_producer_waves,
+                                         int num_consumer_waves, int num_cus, void* stream) {
+    if (!(num_consumer_waves == 4 || num_consumer_waves == 8) || !(tile_dim == 64 || tile_dim == 128 || tile_dim == 256))
+        return ck::CK_ERR_BAD_PARAM;
+    const int mode = ck::sync_mode_of(tile_dim, num_consumer_waves, bar_step_rows_a, bar_step_rows_b);
+    int sa = 0, sb = 0;
+    if (mode == ck::CK_SYNC_WAVE) { sa = num_consumer_waves / 2; sb = 2; }
+    if (mode == ck::CK_SYNC_ACC) {
+        sa = ck::wave_tile_rows(tile_dim, num_consumer_waves) - 1;
+        sb = ck::wave_tile_cols(tile_dim, num_consumer_waves) - 1;
+    }
+    const ck::GemmTuning t{tile_dim, segment_dim_k, sa, sb, bar_step_rows_a, bar_step_rows_b,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream);
+}
+
+int ckopt_gemm_shmem_tc_async_opt_port_0(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                         float alpha, float beta, int M, int N, int K, int tile_dim,
+                                         int segment_dim_k, int tile_group_m, int num_stages,
+                                         int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, 0, 0, tile_dim, tile_dim,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream);
+}
+
+int ckopt_get_lds_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                      int bar_step_rows_b, int num_stages, int num_consumer_waves) {
+    if (!(tile_dim == 64 || tile_dim == 128 || tile_dim == 256) || !(num_consumer_waves == 4 || num_consumer_waves == 8) ||
+        segment_dim_k <= 0 || segment_dim_k % 8 || num_stages < 1 || bar_steps_a < 0 || bar_steps_b < 0)
+        return ck::CK_ERR_BAD_PARAM;
+    const int r = ck::get_lds_req(tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                                  num_stages, num_consumer_waves);
+    return r < 0 ? ck::CK_ERR_BAD_PARAM : r;
+}
+
+int ckopt_get_num_acc(int tile_dim, int num_consumer_waves) {
+    if (!(tile_dim == 64 || tile_dim == 128 || tile_dim == 256) || !(num_consumer_waves == 4 || num_consumer_waves == 8))
+        return ck::CK_ERR_BAD_PARAM;
+    return ck::get_num_acc(tile_dim, num_consumer_waves);
+}
+
+int ckopt_get_warp_tile_rows(int tile_dim, int num_consumer_waves) {
+    if (!(tile_dim == 64 || tile_dim == 128 || tile_dim == 256) || !(num_consumer_waves == 4 || num_consumer_waves == 8))
+        return ck::CK_ERR_BAD_PARAM;
+    return ck::get_warp_tile_rows(tile_dim, num_consumer_waves);
+}
+
+int64_t ckopt_get_tile_offset_cd(int M, int N, int tile_dim, int tile_group_m, int64_t tile_count) {
+    if (M <= 0 || N <= 0 || tile_dim <= 0 || tile_group_m <= 0 || tile_count < 0) return ck::CK_ERR_BAD_PARAM;
+    return ck::get_tile_offset_cd(M, N, tile_dim, tile_group_m, tile_count);
+}
+
+int ckopt_check_gemm_tuning(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b,
+                            int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
+                            int num_producer_waves, int num_consumer_waves, int num_cus) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    return ck::check_gemm_tuning(t);
+}
+
+int ckopt_matmul_shmem(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int tile_dim,
+                       int block_rows, int b_transposed, void* stream) {
+    using namespace ck;
+    if (!(dtype == CK_DT_F32 || dtype == CK_DT_F16 || dtype == CK_DT_I32)) return CK_ERR_BAD_PARAM;
+    const int rc = check_simt_tuning(tile_dim, block_rows);
+    if (rc != CK_OK) return rc;
+    if (M <= 0 || N <= 0 || K <= 0) return CK_ERR_BAD_PARAM;
+    if (M % tile_dim || N % tile_dim || K % SIMT_KT) return CK_ERR_BAD_PARAM;
+    if (!A || !B || !C) return CK_ERR_NULL;
+    if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)C & 3)) return CK_ERR_ALIGNMENT;
+    if (N / tile_dim > 65535) return CK_ERR_TOO_LARGE;
+    SimtArgs a{A, B, C, M, N, K};
+    const hipError_t e = launch_matmul_shmem(dtype, tile_dim, tile_dim / block_rows, b_transposed != 0,
+                                             dim3(M / tile_dim, N / tile_dim), static_cast<hipStream_t>(stream), a);
+    if (e == hipErrorInvalidValue) return CK_ERR_NO_INSTANCE;
+    return e == hipSuccess ? CK_OK : CK_ERR_HIP;
+}
+
+int ckopt_matmul_shmem_lds_req(int dtype, int tile_dim) {
+    if (!(dtype == ck::CK_DT_F32 || dtype == ck::CK_DT_F16 || dtype == ck::CK_DT_I32)) return ck::CK_ERR_BAD_PARAM;
+    if (!(tile_dim == 32 || tile_dim == 64 || tile_dim == 128)) return ck::CK_ERR_BAD_PARAM;
+    return ck::simt_lds_req(tile_dim, 4);
+}
+
+int ckopt_check_matmul_shmem_tuning(int tile_dim, int block_rows) { return ck::check_simt_tuning(tile_dim, block_rows); }
+
+int ckopt_device_status(void* stream) {
+    unsigned int* p = nullptr;
+    const int rc = status_ptr_for_current_device(&p);
+    if (rc != ck::CK_OK) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned int v = 0;
+    if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
+    if (hipMemcpyAsync(&v, p, sizeof(v), hipMemcpyDeviceToHost, s) != hipSuccess) return ck::CK_ERR_HIP;
+    if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
+    if (v != 0) {
+        const unsigned int zero = 0;
+        if (hipMemcpyAsync(p, &zero, sizeof(zero), hipMemcpyHostToDevice, s) != hipSuccess) return ck::CK_ERR_HIP;
+        if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
+    }
+    return (int)(v & 0x7fffffffu);
+}
+
+int ckopt_set_option(int key, int value) {
+    switch (key) {
+        case 0: return g_swizzle.exchange(value != 0);
+        case 1: if (value < 1) return ck::CK_ERR_BAD_PARAM; return g_spin_limit.exchange(value);
+        case 2: if (value < 1 || value > 64) return ck::CK_ERR_BAD_PARAM; return g_num_xcd.exchange(value);
+        default: return ck::CK_ERR_BAD_PARAM;
+    }
+}
+
+const char* ckopt_error_string(int code) {
+    switch (code) {
+        case ck::CK_OK: return "ok";
+        case ck::CK_ERR_BAD_PARAM: return "parameter outside the legal set";
+        case ck::CK_ERR_LDS_BUDGET: return "LDS ring exceeds 160 KiB";
+        case ck::CK_ERR_NO_INSTANCE: return "no kernel instance compiled for this tuple";
+        case ck::CK_ERR_HIP: return "HIP runtime error";
+        case ck::CK_ERR_ALIGNMENT: return "pointer or row pitch misaligned";
+        case ck::CK_ERR_NULL: return "required pointer is NULL";
+        case ck::CK_ERR_TOO_LARGE: return "size exceeds what the entry point supports";
+        default: return "unknown error";
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,4 @@
+#define CK_INST_DT f16_tag
+#define CK_INST_MODE 2
+#define CK_INST_FN launch_gemm_pc_f16_m2
+#include "gemm_pc_inst.inc"

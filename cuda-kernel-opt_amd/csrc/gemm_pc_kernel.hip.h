@@ -1,0 +1,486 @@
+// gemm_shmem_tc_async_opt_port for gfx950: D = alpha * A * Bt^T + beta * C.
+//
+// A is M x K row-major, Bt is N x K row-major (B passed transposed, as the reference does,
+// matmul_shmem_tc_async_opt_port_2.cu:642), both 16-bit (fp16 or bf16); C and D are M x N fp32.
+//
+// One workgroup per CU, persistent over output tiles (reference kernel role: port_2:638-878).
+// Waves [0, PA) stream A K-segments, waves [PA, PA+PB) stream Bt K-segments from HBM/L2 straight
+// into a multi-stage LDS ring with buffer_load ... lds (16 B per lane, no VGPR staging); the
+// remaining CW waves are consumers running v_mfma_f32_16x16x32 into a per-wave accumulator tile of
+// WTR x WTC blocks (the reference's NUM_ACC knob). There is no workgroup barrier in the steady
+// state: producers and consumers meet only through monotonically increasing LDS flag counters.
+//
+//   full  counter: +1 by every producer wave of that operand once its share of the covered rows has
+//                  landed in LDS (s_waitcnt vmcnt(n) on its own in-order load queue, then ds_add).
+//   empty counter: +1 by every consumer wave that has finished reading the covered rows.
+//
+// Counters never reset; the fill number f = global_segment / num_stages gives the expected value
+// (arrivals_per_fill * (f + 1) for full, * f for empty), so the reference's per-tile balancing
+// arrivals (port_2:359-404, :458-482) have no counterpart.
+//
+// Shift synchronisation (port_1 / port_2) maps to the granularity of those counters:
+//   TILE : one full/empty pair per operand and stage.
+//   WAVE : the first bar_steps_a wave-tile rows of A and bar_steps_b wave-tile columns of Bt have
+//          their own counters; consumer waves in that upper-left rectangle start as soon as THEIR
+//          rows and columns have landed. All other waves share one residual counter per operand,
+//          signalled after the last row block.
+//   ACC  : inside every wave tile the first bar_steps_a 16-row blocks of A and bar_steps_b 16-row
+//          blocks of Bt have their own counters; the rest of the wave tile shares a residual one.
+//          The consumer then runs accumulator-outer / k-inner for the early columns.
+#ifndef CK_GEMM_PC_KERNEL_HIP_H
+#define CK_GEMM_PC_KERNEL_HIP_H
+
+#include <hip/hip_runtime.h>
+#include "ck_common.h"
+
+namespace ck {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define CK_LDS __attribute__((address_space(3)))
+
+struct GemmArgs {
+    const void* A;
+    const void* Bt;
+    const float* C;
+    float* D;
+    float alpha, beta;
+    int M, N, K;
+    int tiles_m, tiles_n;
+    int nseg;  // ceil(K / segment_dim_k)
+    int tile_group_m, num_stages;
+    int pa, pb;  // producer waves on A and on Bt
+    int bar_steps_a, bar_steps_b;
+    int swizzle;
+    int num_xcd;
+    int vec_store;  // D (and C) 16-byte aligned with N % 4 == 0
+    uint32_t spin_limit;
+    unsigned int* status;  // device word: OR of CK_STATUS_* bits
+};
+
+enum : unsigned { CK_STATUS_PRODUCER_TIMEOUT = 1u, CK_STATUS_CONSUMER_TIMEOUT = 2u };
+
+struct f16_tag {};
+struct bf16_tag {};
+template <typename T> struct MfmaOp;
+template <> struct MfmaOp<f16_tag> {
+    static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct MfmaOp<bf16_tag> {
+    static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+
+// ---- LDS flag primitives (inline asm so the compiler's wait-count pass does not tie them to the
+// outstanding direct-to-LDS loads and force vmcnt(0) before every flag access) -------------------
+__device__ __forceinline__ uint32_t flag_load(uint32_t lds_addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_addr) : "memory");
+    return __builtin_amdgcn_readfirstlane(v);
+}
+// all earlier LDS reads of this wave have returned before the counter moves
+__device__ __forceinline__ void flag_add_after_reads(uint32_t lds_addr) {
+    uint32_t one = 1;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\tds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
+}
+__device__ __forceinline__ void flag_add(uint32_t lds_addr) {
+    uint32_t one = 1;
+    asm volatile("ds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
+}
+
+template <int N> __device__ __forceinline__ void wait_vmcnt_imm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// wait until at most n of this wave's vector-memory loads are outstanding (n is wave-uniform)
+__device__ __forceinline__ void wait_vmcnt_le(uint32_t n) {
+#define CK_VMCASE(X) case X: wait_vmcnt_imm<X>(); break;
+    switch (n) {
+        CK_VMCASE(0) CK_VMCASE(1) CK_VMCASE(2) CK_VMCASE(3) CK_VMCASE(4) CK_VMCASE(5) CK_VMCASE(6) CK_VMCASE(7)
+        CK_VMCASE(8) CK_VMCASE(9) CK_VMCASE(10) CK_VMCASE(11) CK_VMCASE(12) CK_VMCASE(13) CK_VMCASE(14) CK_VMCASE(15)
+        CK_VMCASE(16) CK_VMCASE(17) CK_VMCASE(18) CK_VMCASE(19) CK_VMCASE(20) CK_VMCASE(21) CK_VMCASE(22) CK_VMCASE(23)
+        CK_VMCASE(24) CK_VMCASE(25) CK_VMCASE(26) CK_VMCASE(27) CK_VMCASE(28) CK_VMCASE(29) CK_VMCASE(30) CK_VMCASE(31)
+        CK_VMCASE(32) CK_VMCASE(33) CK_VMCASE(34) CK_VMCASE(35) CK_VMCASE(36) CK_VMCASE(37) CK_VMCASE(38) CK_VMCASE(39)
+        CK_VMCASE(40) CK_VMCASE(41) CK_VMCASE(42) CK_VMCASE(43) CK_VMCASE(44) CK_VMCASE(45) CK_VMCASE(46) CK_VMCASE(47)
+        default: wait_vmcnt_imm<48>(); break;
+    }
+#undef CK_VMCASE
+}
+
+// Bounded polling: a wave that exceeds the spin limit records a status bit and stops waiting for
+// the rest of the kernel, so every wave reaches the end of the grid whatever goes wrong.
+struct Spin {
+    uint32_t limit;
+    unsigned int* status;
+    unsigned bit;
+    bool dead;
+};
+__device__ __forceinline__ bool flag_ready(uint32_t addr, uint32_t target) { return (int32_t)(flag_load(addr) - target) >= 0; }
+__device__ __forceinline__ void wait_flag_ge(uint32_t addr, uint32_t target, Spin& sp) {
+    if (sp.dead) return;
+    uint32_t n = 0;
+    while (!flag_ready(addr, target)) {
+        if (++n > sp.limit) {
+            sp.dead = true;
+            if ((threadIdx.x & 63) == 0) atomicOr(sp.status, sp.bit);
+            break;
+        }
+        if (n > 4) __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// ---- producer --------------------------------------------------------------------------------------
+// Pending "rows landed" signals of one producer wave: a short in-order queue of (counter address,
+// number of loads issued when the covered rows were complete). Popping entry e needs at most
+// issued_now - e.at loads outstanding, because a wave's loads complete in issue order.
+template <int DEPTH> struct SignalQueue {
+    uint32_t addr[DEPTH];
+    uint32_t at[DEPTH];
+    uint32_t issued;
+    __device__ __forceinline__ void init() {
+#pragma unroll
+        for (int i = 0; i < DEPTH; ++i) { addr[i] = 0; at[i] = 0; }
+        issued = 0;
+    }
+    __device__ __forceinline__ void pop_front() {
+        if (addr[0]) {
+            wait_vmcnt_le(issued - at[0]);
+            flag_add(addr[0] & 0x7fffffffu);
+        }
+#pragma unroll
+        for (int i = 0; i + 1 < DEPTH; ++i) { addr[i] = addr[i + 1]; at[i] = at[i + 1]; }
+        addr[DEPTH - 1] = 0;
+    }
+    __device__ __forceinline__ void push(uint32_t a) {
+        pop_front();  // slot DEPTH-1 is free afterwards
+        addr[DEPTH - 1] = a | 0x80000000u;  // top bit marks the slot as occupied (LDS address 0 is legal)
+        at[DEPTH - 1] = issued;
+    }
+    __device__ __forceinline__ bool pending() const {
+        bool any = false;
+#pragma unroll
+        for (int i = 0; i < DEPTH; ++i) any |= (addr[i] != 0);
+        return any;
+    }
+    __device__ __forceinline__ void drain() {
+        if (!pending()) return;
+        wait_vmcnt_imm<0>();
+#pragma unroll
+        for (int i = 0; i < DEPTH; ++i) {
+            if (addr[i]) flag_add(addr[i] & 0x7fffffffu);
+            addr[i] = 0;
+        }
+    }
+};
+
+// Wait for an "empty" counter. While it is not there yet the wave keeps retiring its own pending
+// "landed" signals oldest first (each needs only the loads up to that entry), so it never blocks
+// while holding back a signal the consumers need to make progress.
+template <int DEPTH>
+__device__ __forceinline__ void producer_wait(uint32_t addr, uint32_t target, SignalQueue<DEPTH>& q, Spin& sp) {
+    if (target == 0 || sp.dead) return;
+    uint32_t n = 0;
+    while (!flag_ready(addr, target)) {
+        if (q.pending()) {
+            q.pop_front();
+            continue;
+        }
+        if (++n > sp.limit) {
+            sp.dead = true;
+            if ((threadIdx.x & 63) == 0) atomicOr(sp.status, sp.bit);
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// IS_A selects the operand: A producers walk wave-tile rows, Bt producers wave-tile columns.
+template <int TILE, int SEGK, int CW, int MODE, bool IS_A>
+__device__ void produce(const GemmArgs& g, uint32_t flags_base, uint32_t ring_base, int q, int px, int lane) {
+    constexpr int WTR = TILE / (CW / 2) / MFMA_M, WTC = TILE / 2 / MFMA_N;
+    constexpr int CPR = SEGK / CHUNK_ELEMS;      // 16-byte chunks per row
+    constexpr int RB = SEGK * 2;                 // row bytes in LDS
+    constexpr int RPI = WAVE / CPR;              // rows one wave load covers
+    constexpr int OPB = TILE * RB;               // bytes of one operand stage
+    constexpr int BLK_ROWS = MODE == CK_SYNC_TILE ? TILE : MODE == CK_SYNC_WAVE ? (IS_A ? WTR : WTC) * 16 : 16;
+    constexpr int NBLK = TILE / BLK_ROWS;
+    constexpr int NIB = BLK_ROWS / RPI;          // wave loads per row block
+    static_assert(BLK_ROWS % RPI == 0, "row block must be whole wave loads");
+
+    const int sa = g.bar_steps_a, sb = g.bar_steps_b;
+    const int S = g.num_stages;
+    const int ua = units_a(MODE, CW, sa), ub = units_b(MODE, CW, sb);
+    const int fps = 2 * ua + 2 * ub;
+    // counters of this operand inside one stage's flag set
+    const uint32_t full_off = IS_A ? 0 : 2 * ua;
+    const uint32_t empty_off = IS_A ? ua : 2 * ua + ub;
+    const int nres = CW - sa * sb;  // WAVE mode: consumer waves on the residual counters
+
+    const char* base = (const char*)(IS_A ? g.A : g.Bt);
+    const int rows_total = IS_A ? g.M : g.N;
+    const int64_t pitch = (int64_t)g.K * 2;
+
+    const int lane_row = lane / CPR, lane_slot = lane % CPR;
+    const int grid = gridDim.x;
+    const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
+    const int64_t total_tiles = (int64_t)g.tiles_m * g.tiles_n;
+
+    Spin sp{g.spin_limit, g.status, CK_STATUS_PRODUCER_TIMEOUT, false};
+    SignalQueue<MODE == CK_SYNC_TILE ? 3 : MODE == CK_SYNC_WAVE ? 4 : 8> sq;
+    sq.init();
+
+    int stage = 0;
+    uint32_t fill = 0;
+    for (int64_t tc = slot; tc < total_tiles; tc += grid) {
+        const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
+        const int row0 = (IS_A ? rc.row : rc.col) * TILE;
+        int rows_here = rows_total - row0;
+        rows_here = rows_here < TILE ? rows_here : TILE;
+        const uint32_t num_records = (uint32_t)((int64_t)rows_here * pitch);
+        __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)row0 * pitch), 0, (int)num_records, 0x00020000);
+
+        for (int seg = 0; seg < g.nseg; ++seg) {
+            const uint32_t fl = flags_base + (uint32_t)stage * fps * 4;
+            const uint32_t st_base = ring_base + (uint32_t)stage * (2 * OPB) + (IS_A ? 0 : OPB);
+            const int k0 = seg * SEGK;
+#pragma unroll 1
+            for (int blk = 0; blk < NBLK; ++blk) {
+                // ---- wait until the consumers of the previous fill have released these rows
+                if (MODE == CK_SYNC_TILE) {
+                    producer_wait(fl + (empty_off + 0) * 4, CW * fill, sq, sp);
+                } else if (MODE == CK_SYNC_WAVE) {
+                    const int s_own = IS_A ? sa : sb, s_oth = IS_A ? sb : sa;
+                    const int oth_max = IS_A ? 2 : CW / 2;
+                    const bool first_has_res = (s_own == 0 || s_oth < oth_max);
+                    if (blk == 0 && first_has_res && nres > 0) producer_wait(fl + (empty_off + s_own) * 4, nres * fill, sq, sp);
+                    if (blk < s_own && s_oth > 0) {
+                        producer_wait(fl + (empty_off + blk) * 4, s_oth * fill, sq, sp);
+                    } else if (blk == s_own && !first_has_res && nres > 0) {
+                        producer_wait(fl + (empty_off + s_own) * 4, nres * fill, sq, sp);
+                    }
+                } else {
+                    constexpr int WT = IS_A ? WTR : WTC;
+                    const int s_own = IS_A ? sa : sb;
+                    const int unit = blk / WT, sub = blk % WT;
+                    const int readers = IS_A ? 2 : CW / 2;
+                    if (sub <= s_own) producer_wait(fl + (empty_off + unit * (s_own + 1) + sub) * 4, readers * fill, sq, sp);
+                }
+                // ---- this wave's share of the row block, straight into LDS
+#pragma unroll
+                for (int e = 0; e < NIB; ++e) {
+                    const int E = blk * NIB + e;
+                    if (E % px != q) continue;
+                    const int r = E * RPI + lane_row;
+                    const int c = swizzle_slot(r, lane_slot, CPR, g.swizzle);  // logical chunk stored at this slot
+                    const int k = k0 + c * CHUNK_ELEMS;
+                    uint32_t voff = (uint32_t)r * (uint32_t)pitch + (uint32_t)k * 2u;
+                    if (k >= g.K) voff = num_records;  // out of range: the load writes zeros
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (CK_LDS void*)(uintptr_t)(st_base + (uint32_t)E * 1024u), 16, voff, 0, 0, 0);
+                    sq.issued++;
+                }
+                // ---- queue the "landed" signals this block completes
+                if (MODE == CK_SYNC_TILE) {
+                    sq.push(fl + (full_off + 0) * 4);
+                } else if (MODE == CK_SYNC_WAVE) {
+                    const int s_own = IS_A ? sa : sb;
+                    if (blk < s_own) sq.push(fl + (full_off + blk) * 4);
+                    if (blk == NBLK - 1) sq.push(fl + (full_off + s_own) * 4);
+                } else {
+                    constexpr int WT = IS_A ? WTR : WTC;
+                    const int s_own = IS_A ? sa : sb;
+                    const int unit = blk / WT, sub = blk % WT;
+                    if (sub < s_own) sq.push(fl + (full_off + unit * (s_own + 1) + sub) * 4);
+                    else if (sub == WT - 1) sq.push(fl + (full_off + unit * (s_own + 1) + s_own) * 4);
+                }
+            }
+            if (++stage == S) { stage = 0; ++fill; }
+        }
+    }
+    sq.drain();
+}
+
+// ---- consumer ----------------------------------------------------------------------------------------
+template <typename DT, int TILE, int SEGK, int CW, int MODE>
+__device__ void consume(const GemmArgs& g, uint32_t flags_base, uint32_t ring_base, int cw, int lane) {
+    constexpr int WTR = TILE / (CW / 2) / MFMA_M, WTC = TILE / 2 / MFMA_N;
+    constexpr int CPR = SEGK / CHUNK_ELEMS;
+    constexpr int RB = SEGK * 2;
+    constexpr int OPB = TILE * RB;
+    constexpr int KSTEPS = SEGK / MFMA_K;
+
+    const int sa = g.bar_steps_a, sb = g.bar_steps_b;
+    const int S = g.num_stages;
+    const int ua = units_a(MODE, CW, sa), ub = units_b(MODE, CW, sb);
+    const int fps = 2 * ua + 2 * ub;
+    const int R = cw / 2, Cc = cw % 2;  // wave-tile row / column of this wave
+    const uint32_t pa = g.pa, pb = g.pb;
+
+    // lane -> fragment element: row (lane % 16) of a 16-row block, logical chunk kstep*4 + lane/16
+    const int lr = lane & 15, lg = lane >> 4;
+    const int key = g.swizzle ? swizzle_key(lr, CPR) : 0;  // same for every 16-row block
+    const uint32_t a_lane = (uint32_t)(R * WTR * 16 + lr) * RB;
+    const uint32_t b_lane = (uint32_t)OPB + (uint32_t)(Cc * WTC * 16 + lr) * RB;
+
+    const int grid = gridDim.x;
+    const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
+    const int64_t total_tiles = (int64_t)g.tiles_m * g.tiles_n;
+    Spin sp{g.spin_limit, g.status, CK_STATUS_CONSUMER_TIMEOUT, false};
+
+    // WAVE mode: which counters this wave uses
+    const bool individual = (MODE == CK_SYNC_WAVE) && R < sa && Cc < sb;
+    int fa_idx = 0, fb_idx = 0;
+    if (MODE == CK_SYNC_WAVE) { fa_idx = individual ? R : sa; fb_idx = individual ? Cc : sb; }
+
+    int stage = 0;
+    uint32_t fill = 0;
+    for (int64_t tc = slot; tc < total_tiles; tc += grid) {
+        const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
+        f32x4 acc[WTR][WTC];
+#pragma unroll
+        for (int i = 0; i < WTR; ++i)
+#pragma unroll
+            for (int j = 0; j < WTC; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        for (int seg = 0; seg < g.nseg; ++seg) {
+            const uint32_t fl = flags_base + (uint32_t)stage * fps * 4;
+            const uint32_t st = ring_base + (uint32_t)stage * (2 * OPB);
+            const uint32_t fullA = fl, emptyA = fl + ua * 4, fullB = fl + 2 * ua * 4, emptyB = fl + (2 * ua + ub) * 4;
+
+            if (MODE != CK_SYNC_ACC) {
+                wait_flag_ge(fullA + fa_idx * 4, pa * (fill + 1), sp);
+                wait_flag_ge(fullB + fb_idx * 4, pb * (fill + 1), sp);
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks) {
+                    const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
+                    u32x4 a[WTR], b[WTC];
+#pragma unroll
+                    for (int i = 0; i < WTR; ++i) a[i] = *(const CK_LDS u32x4*)(uintptr_t)(st + a_lane + coff + i * 16 * RB);
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j) b[j] = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + j * 16 * RB);
+                    if (ks == KSTEPS - 1) {
+                        flag_add_after_reads(emptyA + fa_idx * 4);
+                        flag_add(emptyB + fb_idx * 4);
+                    }
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j)
+#pragma unroll
+                        for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(b[j], a[i], acc[i][j]);
+                }
+            } else {
+                // accumulator granularity: counters per (wave-tile row, 16-row block) and per
+                // (wave-tile column, 16-row block); early columns run accumulator-outer, k-inner
+                const uint32_t fa = fullA + R * (sa + 1) * 4, ea = emptyA + R * (sa + 1) * 4;
+                const uint32_t fb = fullB + Cc * (sb + 1) * 4, eb = emptyB + Cc * (sb + 1) * 4;
+                int a_waited = -1;  // highest A counter index already waited for in this segment
+                // phase 1: every row against the first sb columns
+#pragma unroll
+                for (int i = 0; i < WTR; ++i) {
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j) {
+                        if (j < sb) {
+                            const int ai = i < sa ? i : sa;
+                            if (ai > a_waited) { wait_flag_ge(fa + ai * 4, pa * (fill + 1), sp); a_waited = ai; }
+                            if (i == 0) wait_flag_ge(fb + j * 4, pb * (fill + 1), sp);
+#pragma unroll
+                            for (int ks = 0; ks < KSTEPS; ++ks) {
+                                const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
+                                const u32x4 av = *(const CK_LDS u32x4*)(uintptr_t)(st + a_lane + coff + i * 16 * RB);
+                                const u32x4 bv = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + j * 16 * RB);
+                                acc[i][j] = MfmaOp<DT>::run(bv, av, acc[i][j]);
+                            }
+                            if (i == WTR - 1) flag_add_after_reads(eb + j * 4);
+                        }
+                    }
+                }
+                // phase 2: every row against the residual columns
+                wait_flag_ge(fb + sb * 4, pb * (fill + 1), sp);
+#pragma unroll
+                for (int i = 0; i < WTR; ++i) {
+                    const int ai = i < sa ? i : sa;
+                    if (ai > a_waited) { wait_flag_ge(fa + ai * 4, pa * (fill + 1), sp); a_waited = ai; }
+                    u32x4 a[KSTEPS];
+#pragma unroll
+                    for (int ks = 0; ks < KSTEPS; ++ks) {
+                        const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
+                        a[ks] = *(const CK_LDS u32x4*)(uintptr_t)(st + a_lane + coff + i * 16 * RB);
+                    }
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j) {
+                        if (j >= sb) {
+#pragma unroll
+                            for (int ks = 0; ks < KSTEPS; ++ks) {
+                                const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
+                                const u32x4 bv = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + j * 16 * RB);
+                                acc[i][j] = MfmaOp<DT>::run(bv, a[ks], acc[i][j]);
+                            }
+                        }
+                    }
+                    if (i < sa) flag_add_after_reads(ea + i * 4);
+                    if (i == WTR - 1) {
+                        flag_add_after_reads(ea + sa * 4);
+                        flag_add(eb + sb * 4);
+                    }
+                }
+            }
+            if (++stage == S) { stage = 0; ++fill; }
+        }
+
+        // ---- epilogue: D = alpha * acc + beta * C straight from the accumulators. With the Bt
+        // fragment as the first MFMA operand a lane holds 4 consecutive columns of one row.
+        const int m_base = rc.row * TILE + R * WTR * 16 + lr;
+        const int n_base = rc.col * TILE + Cc * WTC * 16 + lg * 4;
+        const float alpha = g.alpha, beta = g.beta;
+        const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
+#pragma unroll
+        for (int i = 0; i < WTR; ++i) {
+            const int m = m_base + i * 16;
+#pragma unroll
+            for (int j = 0; j < WTC; ++j) {
+                const int n = n_base + j * 16;
+                const int64_t off = (int64_t)m * g.N + n;
+                f32x4 v = acc[i][j] * alpha;
+                if (interior) {
+                    if (beta != 0.f) v += *(const f32x4*)(g.C + off) * beta;
+                    *(f32x4*)(g.D + off) = v;
+                } else if (m < g.M) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (n + e < g.N) {
+                            float x = v[e];
+                            if (beta != 0.f) x += g.C[off + e] * beta;
+                            g.D[off + e] = x;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename DT, int TILE, int SEGK, int CW, int MODE, int MAXW>
+__global__ __launch_bounds__(MAXW * 64) void gemm_pc_kernel(const GemmArgs g) {
+    extern __shared__ __attribute__((aligned(1024))) char ck_smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(CK_LDS char*)ck_smem;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+
+    const int fregion = flag_region_bytes(MODE, CW, g.bar_steps_a, g.bar_steps_b, g.num_stages);
+    for (int i = threadIdx.x; i < fregion / 4; i += blockDim.x) ((CK_LDS uint32_t*)ck_smem)[i] = 0;
+    __syncthreads();
+
+    const uint32_t flags_base = lds0, ring_base = lds0 + fregion;
+    if (wave < g.pa) {
+        produce<TILE, SEGK, CW, MODE, true>(g, flags_base, ring_base, wave, g.pa, lane);
+    } else if (wave < g.pa + g.pb) {
+        produce<TILE, SEGK, CW, MODE, false>(g, flags_base, ring_base, wave - g.pa, g.pb, lane);
+    } else if (wave < g.pa + g.pb + CW) {
+        consume<DT, TILE, SEGK, CW, MODE>(g, flags_base, ring_base, wave - g.pa - g.pb, lane);
+    }
+}
+
+}  // namespace ck
+#endif  // CK_GEMM_PC_KERNEL_HIP_H

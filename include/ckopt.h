@@ -1,0 +1,126 @@
+/* C ABI of the MI355X (gfx950) GEMM hot path: the drop-in boundary.
+ *
+ * The reference has no FFI; its boundary is one C++ host launcher template per translation unit.
+ * Each entry point below replaces one of those launchers and keeps its parameter order and
+ * meaning. Differences that hold for every entry point:
+ *   - element types are selected by an int (CKOPT_DT_*) instead of template arguments;
+ *   - the return value is 0 or a negative CKOPT_ERR_* code where the reference asserts or swallows
+ *     the error (matmul_shmem_tc_async_opt_port_2.cu:76-85, :1112-1123);
+ *   - a trailing `stream` (a hipStream_t passed as void*, NULL = default stream) is added;
+ *   - "warps" are 64-lane wavefronts and "SMs" are compute units.
+ * All pointers are device memory owned by the caller. Nothing is allocated, freed or
+ * synchronised; launches are asynchronous on `stream`.
+ */
+#ifndef CKOPT_H
+#define CKOPT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { CKOPT_DT_F16 = 0, CKOPT_DT_BF16 = 1, CKOPT_DT_F32 = 2, CKOPT_DT_I32 = 3 };
+
+enum {
+    CKOPT_OK = 0,
+    CKOPT_ERR_BAD_PARAM = -1,   /* tuning or shape parameter outside the legal set */
+    CKOPT_ERR_LDS_BUDGET = -2,  /* ring does not fit 160 KiB of LDS */
+    CKOPT_ERR_NO_INSTANCE = -3, /* legal, but no kernel instance is compiled for the tuple */
+    CKOPT_ERR_HIP = -4,         /* a HIP runtime call failed */
+    CKOPT_ERR_ALIGNMENT = -5,   /* pointer or row pitch not aligned as required */
+    CKOPT_ERR_NULL = -6,        /* required pointer is NULL */
+    CKOPT_ERR_TOO_LARGE = -7    /* size beyond what the entry point supports */
+};
+
+/* Replaces gemm_shmem_tc_async_opt_port<DT,DT_ACC>() of matmul_shmem_tc_async_opt_port_2.cu:1088-1168.
+ * D = alpha * A * Bt^T + beta * C (textbook form; C is not read when beta == 0).
+ * A: M x K row-major, Bt: N x K row-major (B transposed), dtype CKOPT_DT_F16 or CKOPT_DT_BF16;
+ * C, D: M x N row-major fp32, distinct buffers (C may be NULL when beta == 0).
+ * tile_dim in {64,128,256}; segment_dim_k in {32,64,128}; bar_step_rows_{a,b} select the
+ * synchronisation granularity exactly as in the reference: (tile_dim, tile_dim), or
+ * (wave_tile_rows*16, wave_tile_cols*16) with bar_steps_a <= C/2 and bar_steps_b <= 2, or (16, 16)
+ * with bar_steps_a < wave_tile_rows and bar_steps_b < wave_tile_cols; num_producer_waves in
+ * {2,4,8} (half stream A, half stream Bt); num_consumer_waves in {4,8}; num_cus = persistent grid.
+ * M, N need not be multiples of tile_dim and K need not be a multiple of segment_dim_k (edges are
+ * zero-filled / masked), but K must be a multiple of 8 so that rows are 16-byte aligned. */
+int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                         float alpha, float beta, int M, int N, int K, int tile_dim,
+                                         int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                                         int bar_step_rows_b, int tile_group_m, int num_stages,
+                                         int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
+
+/* Replaces gemm_shmem_tc_async_opt_port<DT,DT_ACC>() of matmul_shmem_tc_async_opt_port_1.cu:889-965:
+ * every wave tile (or every 16-row block) has its own signal, i.e. port_2 with maximal bar_steps. */
+int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                         float alpha, float beta, int M, int N, int K, int tile_dim,
+                                         int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
+                                         int tile_group_m, int num_stages, int num_producer_waves,
+                                         int num_consumer_waves, int num_cus, void* stream);
+
+/* Replaces gemm_shmem_tc_async_opt_port<DT,DT_ACC>() of matmul_shmem_tc_async_opt_port_0.cu:515-579:
+ * one full/empty signal pair per operand and stage. */
+int ckopt_gemm_shmem_tc_async_opt_port_0(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                         float alpha, float beta, int M, int N, int K, int tile_dim,
+                                         int segment_dim_k, int tile_group_m, int num_stages,
+                                         int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
+
+/* Role of get_shmem_req<DT,DT_ACC>() (port_2.cu:1057-1086): dynamic LDS bytes of the launch, or a
+ * negative error code. The caller may compare it with 160 KiB; the launcher does so itself. */
+int ckopt_get_lds_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                      int bar_step_rows_b, int num_stages, int num_consumer_waves);
+
+/* get_num_acc / get_warp_tile_rows (port_2.cu:158-169), extended to tile_dim 256. */
+int ckopt_get_num_acc(int tile_dim, int num_consumer_waves);
+int ckopt_get_warp_tile_rows(int tile_dim, int num_consumer_waves);
+
+/* get_tile_offset_cd (port_2.cu:605-614) with 64-bit offsets and ceil-divided tile counts. */
+int64_t ckopt_get_tile_offset_cd(int M, int N, int tile_dim, int tile_group_m, int64_t tile_count);
+
+/* Validates a port_2 tuning tuple without launching (the reference's asserts, port_2.cu:1112-1123,
+ * plus the LDS budget and the instance table). Returns CKOPT_OK or the error the launch would give. */
+int ckopt_check_gemm_tuning(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b,
+                            int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
+                            int num_producer_waves, int num_consumer_waves, int num_cus);
+
+/* Replaces matmul_shmem<DT,DT_ACC>() of matmul_shmem.cu:143-174: C = A * B without matrix cores.
+ * dtype CKOPT_DT_F32 (fp32 in, fp32 accumulate), CKOPT_DT_F16 (fp16 in/out, fp32 accumulate) or
+ * CKOPT_DT_I32 (exact). A: M x K, C: M x N row-major. b_transposed == 0: B is K x N row-major as in
+ * the reference; b_transposed != 0: B is given as N x K row-major.
+ * tile_dim in {32,64,128}, tile_dim % block_rows == 0, accumulators per thread
+ * tile_dim/block_rows in {1,2,4,8,16,32,64}, 64 <= tile_dim*block_rows <= 1024.
+ * M, N must be multiples of tile_dim and K a multiple of 16. */
+int ckopt_matmul_shmem(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int tile_dim,
+                       int block_rows, int b_transposed, void* stream);
+
+/* Role of get_shmem_req<DT>(tile_dim) (matmul_shmem.cu:138-141). */
+int ckopt_matmul_shmem_lds_req(int dtype, int tile_dim);
+int ckopt_check_matmul_shmem_tuning(int tile_dim, int block_rows);
+
+/* Waits for `stream`, then returns the device status word of the current device and clears it:
+ * 0 = all flag waits inside the GEMM kernels completed; bit 0 / bit 1 = a producer / consumer wave
+ * gave up a bounded wait (results are then invalid). Negative = HIP error. No reference counterpart
+ * (cuda::barrier waits are unbounded). */
+int ckopt_device_status(void* stream);
+
+/* Process-wide tuning switches that are not launcher parameters in the reference:
+ * key 0: LDS XOR swizzle on/off (default 1); key 1: spin limit of bounded waits (default 1<<22);
+ * key 2: number of XCDs assumed by the workgroup->tile remap (default 8; 1 disables the remap).
+ * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
+int ckopt_set_option(int key, int value);
+
+/* Seeded host-side input generation (role of MatmulTest*::Rerand / SetConstant, matmul_test.h:160-168,
+ * :328-351). Element i of stream `stream_id` depends only on (seed, stream_id, i): value i is the
+ * (i+1)-th output of SplitMix64 started at seed + stream_id * 0xD1342543DE82EF95, reduced to a
+ * 24-bit uniform in [0,1). `out` is HOST memory of n elements of `dtype`. */
+int ckopt_fill_uniform(int dtype, void* out, int64_t n, uint64_t seed, uint64_t stream_id, float lo, float hi);
+int ckopt_fill_normal(int dtype, void* out, int64_t n, uint64_t seed, uint64_t stream_id, float mean, float stddev);
+int ckopt_fill_int(int dtype, void* out, int64_t n, uint64_t seed, uint64_t stream_id, int lo, int hi_inclusive);
+int ckopt_fill_constant(int dtype, void* out, int64_t n, float value);
+
+const char* ckopt_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CKOPT_H */
