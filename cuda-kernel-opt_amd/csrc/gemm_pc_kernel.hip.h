@@ -84,14 +84,20 @@ __device__ __forceinline__ uint32_t flag_load(uint32_t lds_addr) {
     asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_addr) : "memory");
     return __builtin_amdgcn_readfirstlane(v);
 }
+// Counters move by exactly 1 per wave: only lane 0 issues the LDS atomic.
 // all earlier LDS reads of this wave have returned before the counter moves
 __device__ __forceinline__ void flag_add_after_reads(uint32_t lds_addr) {
-    uint32_t one = 1;
-    asm volatile("s_waitcnt lgkmcnt(0)\n\tds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if ((threadIdx.x & 63) == 0) {
+        uint32_t one = 1;
+        asm volatile("ds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
+    }
 }
 __device__ __forceinline__ void flag_add(uint32_t lds_addr) {
-    uint32_t one = 1;
-    asm volatile("ds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
+    if ((threadIdx.x & 63) == 0) {
+        uint32_t one = 1;
+        asm volatile("ds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
+    }
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt_imm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
