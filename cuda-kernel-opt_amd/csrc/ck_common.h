@@ -103,8 +103,9 @@ CK_HD int xcd_slot(int block, int grid, int num_xcd) {
 // logical chunk) fall into 16 distinct 4-bank groups of the 64-bank LDS.
 CK_HD int chunks_per_row(int segment_dim_k) { return segment_dim_k / CHUNK_ELEMS; }
 CK_HD int swizzle_key(int row, int cpr) {
-    // cpr in {4, 8, 16}: rows per 256-byte bank line = 16 / cpr
-    return (row / (16 / cpr)) % cpr;
+    // Found conflict-free for ds_read_b128 on gfx950 by measurement (64 banks, 256 B/clk): rows of
+    // 64 and 128 bytes rotate with every second row, rows of 256 bytes with every row.
+    return cpr == 16 ? row % 16 : (row >> 1) % cpr;
 }
 // slot (physical chunk index inside the row) that holds logical chunk c of row `row`
 CK_HD int swizzle_slot(int row, int c, int cpr, int swizzle_on) { return swizzle_on ? (c ^ swizzle_key(row, cpr)) : c; }

@@ -84,36 +84,36 @@ __device__ __forceinline__ uint32_t flag_load(uint32_t lds_addr) {
     asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_addr) : "memory");
     return __builtin_amdgcn_readfirstlane(v);
 }
-// Counters move by exactly 1 per wave: only lane 0 issues the LDS atomic.
+// Counters move by exactly 1 per wave: the LDS atomic is issued with only lane 0 enabled. The
+// EXEC mask is narrowed and restored inside one asm block; every caller runs with all 64 lanes
+// active (no lane-divergent control flow in producers or consumers), so restoring to all ones is
+// restoring the caller's mask.
 // all earlier LDS reads of this wave have returned before the counter moves
 __device__ __forceinline__ void flag_add_after_reads(uint32_t lds_addr) {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if ((threadIdx.x & 63) == 0) {
-        uint32_t one = 1;
-        asm volatile("ds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
-    }
+    uint32_t one = 1;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_mov_b64 exec, 1\n\tds_add_u32 %0, %1\n\ts_mov_b64 exec, -1" ::"v"(lds_addr), "v"(one) : "memory");
 }
 __device__ __forceinline__ void flag_add(uint32_t lds_addr) {
-    if ((threadIdx.x & 63) == 0) {
-        uint32_t one = 1;
-        asm volatile("ds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
-    }
+    uint32_t one = 1;
+    asm volatile("s_mov_b64 exec, 1\n\tds_add_u32 %0, %1\n\ts_mov_b64 exec, -1" ::"v"(lds_addr), "v"(one) : "memory");
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt_imm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-// wait until at most n of this wave's vector-memory loads are outstanding (n is wave-uniform)
+// wait until at most n of this wave's vector-memory loads are outstanding (n is wave-uniform);
+// the immediate is the largest rung not above n, so the wait is exact or slightly early-safe
 __device__ __forceinline__ void wait_vmcnt_le(uint32_t n) {
-#define CK_VMCASE(X) case X: wait_vmcnt_imm<X>(); break;
-    switch (n) {
-        CK_VMCASE(0) CK_VMCASE(1) CK_VMCASE(2) CK_VMCASE(3) CK_VMCASE(4) CK_VMCASE(5) CK_VMCASE(6) CK_VMCASE(7)
-        CK_VMCASE(8) CK_VMCASE(9) CK_VMCASE(10) CK_VMCASE(11) CK_VMCASE(12) CK_VMCASE(13) CK_VMCASE(14) CK_VMCASE(15)
-        CK_VMCASE(16) CK_VMCASE(17) CK_VMCASE(18) CK_VMCASE(19) CK_VMCASE(20) CK_VMCASE(21) CK_VMCASE(22) CK_VMCASE(23)
-        CK_VMCASE(24) CK_VMCASE(25) CK_VMCASE(26) CK_VMCASE(27) CK_VMCASE(28) CK_VMCASE(29) CK_VMCASE(30) CK_VMCASE(31)
-        CK_VMCASE(32) CK_VMCASE(33) CK_VMCASE(34) CK_VMCASE(35) CK_VMCASE(36) CK_VMCASE(37) CK_VMCASE(38) CK_VMCASE(39)
-        CK_VMCASE(40) CK_VMCASE(41) CK_VMCASE(42) CK_VMCASE(43) CK_VMCASE(44) CK_VMCASE(45) CK_VMCASE(46) CK_VMCASE(47)
-        default: wait_vmcnt_imm<48>(); break;
-    }
-#undef CK_VMCASE
+    if (n >= 48) wait_vmcnt_imm<48>();
+    else if (n >= 32) wait_vmcnt_imm<32>();
+    else if (n >= 24) wait_vmcnt_imm<24>();
+    else if (n >= 16) wait_vmcnt_imm<16>();
+    else if (n >= 12) wait_vmcnt_imm<12>();
+    else if (n >= 8) wait_vmcnt_imm<8>();
+    else if (n >= 6) wait_vmcnt_imm<6>();
+    else if (n >= 4) wait_vmcnt_imm<4>();
+    else if (n == 3) wait_vmcnt_imm<3>();
+    else if (n == 2) wait_vmcnt_imm<2>();
+    else if (n == 1) wait_vmcnt_imm<1>();
+    else wait_vmcnt_imm<0>();
 }
 
 // Bounded polling: a wave that exceeds the spin limit records a status bit and stops waiting for
@@ -204,8 +204,19 @@ __device__ __forceinline__ void producer_wait(uint32_t addr, uint32_t target, Si
 }
 
 // IS_A selects the operand: A producers walk wave-tile rows, Bt producers wave-tile columns.
-template <int TILE, int SEGK, int CW, int MODE, bool IS_A>
-__device__ void produce(const GemmArgs& g, uint32_t flags_base, uint32_t ring_base, int q, int px, int lane) {
+// PX = producer waves on this operand; wave q issues the wave loads E with E % PX == q.
+//
+// Address generation is kept off the vector ALU. A wave load E covers rows [E*RPI, (E+1)*RPI) of
+// the operand stage; lane (lane_row, lane_slot) fetches the 16-byte chunk that belongs at its
+// linear LDS slot under the XOR swizzle. The swizzle key of a lane repeats with period VAR in E,
+// so VAR per-lane byte offsets (row-in-load * pitch + chunk * 16) are computed once per kernel and
+// everything that changes from load to load (E * RPI * pitch), from segment to segment (k0 * 2)
+// and from tile to tile (the buffer base) is scalar: the load's soffset, M0 and the descriptor.
+// The scalar offset is not range-checked by the buffer unit, so that fast path is taken only when
+// all rows of the tile and all k of the segment exist; edge tiles and the K tail put the whole
+// offset in the range-checked vector offset and push absent k out of range (zero fill).
+template <int TILE, int SEGK, int CW, int MODE, bool IS_A, int PX>
+__device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, uint32_t ring_base, int q, int lane) {
     constexpr int WTR = TILE / (CW / 2) / MFMA_M, WTC = TILE / 2 / MFMA_N;
     constexpr int CPR = SEGK / CHUNK_ELEMS;      // 16-byte chunks per row
     constexpr int RB = SEGK * 2;                 // row bytes in LDS
@@ -214,6 +225,7 @@ __device__ void produce(const GemmArgs& g, uint32_t flags_base, uint32_t ring_ba
     constexpr int BLK_ROWS = MODE == CK_SYNC_TILE ? TILE : MODE == CK_SYNC_WAVE ? (IS_A ? WTR : WTC) * 16 : 16;
     constexpr int NBLK = TILE / BLK_ROWS;
     constexpr int NIB = BLK_ROWS / RPI;          // wave loads per row block
+    constexpr int VAR = CPR == 4 ? 1 : CPR == 8 ? 2 : 4;  // period of the swizzle key in E
     static_assert(BLK_ROWS % RPI == 0, "row block must be whole wave loads");
 
     const int sa = g.bar_steps_a, sb = g.bar_steps_b;
@@ -228,8 +240,18 @@ __device__ void produce(const GemmArgs& g, uint32_t flags_base, uint32_t ring_ba
     const char* base = (const char*)(IS_A ? g.A : g.Bt);
     const int rows_total = IS_A ? g.M : g.N;
     const int64_t pitch = (int64_t)g.K * 2;
+    const uint32_t pitch32 = (uint32_t)pitch;
 
     const int lane_row = lane / CPR, lane_slot = lane % CPR;
+    uint32_t lane_off[VAR];  // row-in-load * pitch + logical chunk * 16, per swizzle-key variant
+    int lane_chunk[VAR];
+#pragma unroll
+    for (int v = 0; v < VAR; ++v) {
+        lane_chunk[v] = swizzle_slot(v * RPI + lane_row, lane_slot, CPR, g.swizzle);
+        lane_off[v] = (uint32_t)lane_row * pitch32 + (uint32_t)lane_chunk[v] * CHUNK_BYTES;
+    }
+    const uint32_t load_step = (uint32_t)RPI * pitch32;  // bytes between consecutive wave loads
+
     const int grid = gridDim.x;
     const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
     const int64_t total_tiles = (int64_t)g.tiles_m * g.tiles_n;
@@ -242,18 +264,23 @@ __device__ void produce(const GemmArgs& g, uint32_t flags_base, uint32_t ring_ba
     uint32_t fill = 0;
     for (int64_t tc = slot; tc < total_tiles; tc += grid) {
         const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
-        const int row0 = (IS_A ? rc.row : rc.col) * TILE;
+        const int row0 = __builtin_amdgcn_readfirstlane((IS_A ? rc.row : rc.col) * TILE);
         int rows_here = rows_total - row0;
         rows_here = rows_here < TILE ? rows_here : TILE;
         const uint32_t num_records = (uint32_t)((int64_t)rows_here * pitch);
         __amdgpu_buffer_rsrc_t rsrc =
             __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)row0 * pitch), 0, (int)num_records, 0x00020000);
+        const bool all_rows = rows_here == TILE;
 
         for (int seg = 0; seg < g.nseg; ++seg) {
+            // loop-carried scalars are pinned to SGPRs so that address and flag arithmetic stays scalar
+            stage = __builtin_amdgcn_readfirstlane(stage);
+            fill = __builtin_amdgcn_readfirstlane(fill);
             const uint32_t fl = flags_base + (uint32_t)stage * fps * 4;
             const uint32_t st_base = ring_base + (uint32_t)stage * (2 * OPB) + (IS_A ? 0 : OPB);
             const int k0 = seg * SEGK;
-#pragma unroll 1
+            const bool fast = all_rows && k0 + SEGK <= g.K;
+#pragma unroll
             for (int blk = 0; blk < NBLK; ++blk) {
                 // ---- wait until the consumers of the previous fill have released these rows
                 if (MODE == CK_SYNC_TILE) {
@@ -276,17 +303,26 @@ __device__ void produce(const GemmArgs& g, uint32_t flags_base, uint32_t ring_ba
                     if (sub <= s_own) producer_wait(fl + (empty_off + unit * (s_own + 1) + sub) * 4, readers * fill, sq, sp);
                 }
                 // ---- this wave's share of the row block, straight into LDS
+                if (fast) {
+                    const uint32_t soff0 = (uint32_t)k0 * 2u;
 #pragma unroll
-                for (int e = 0; e < NIB; ++e) {
-                    const int E = blk * NIB + e;
-                    if (E % px != q) continue;
-                    const int r = E * RPI + lane_row;
-                    const int c = swizzle_slot(r, lane_slot, CPR, g.swizzle);  // logical chunk stored at this slot
-                    const int k = k0 + c * CHUNK_ELEMS;
-                    uint32_t voff = (uint32_t)r * (uint32_t)pitch + (uint32_t)k * 2u;
-                    if (k >= g.K) voff = num_records;  // out of range: the load writes zeros
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (CK_LDS void*)(uintptr_t)(st_base + (uint32_t)E * 1024u), 16, voff, 0, 0, 0);
-                    sq.issued++;
+                    for (int e = 0; e < NIB; ++e) {
+                        const int E = blk * NIB + e;
+                        if (PX > 1 && E % PX != q) continue;
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (CK_LDS void*)(uintptr_t)(st_base + (uint32_t)E * 1024u), 16,
+                                                                 lane_off[E % VAR], soff0 + (uint32_t)E * load_step, 0, 0);
+                        sq.issued++;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < NIB; ++e) {
+                        const int E = blk * NIB + e;
+                        if (PX > 1 && E % PX != q) continue;
+                        uint32_t voff = lane_off[E % VAR] + (uint32_t)E * load_step + (uint32_t)k0 * 2u;
+                        if (k0 + lane_chunk[E % VAR] * CHUNK_ELEMS >= g.K) voff = num_records;  // absent k: zero fill
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (CK_LDS void*)(uintptr_t)(st_base + (uint32_t)E * 1024u), 16, voff, 0, 0, 0);
+                        sq.issued++;
+                    }
                 }
                 // ---- queue the "landed" signals this block completes
                 if (MODE == CK_SYNC_TILE) {
@@ -309,9 +345,16 @@ __device__ void produce(const GemmArgs& g, uint32_t flags_base, uint32_t ring_ba
     sq.drain();
 }
 
+template <int TILE, int SEGK, int CW, int MODE, bool IS_A>
+__device__ __forceinline__ void produce_px(const GemmArgs& g, uint32_t flags_base, uint32_t ring_base, int q, int px, int lane) {
+    if (px == 1) produce<TILE, SEGK, CW, MODE, IS_A, 1>(g, flags_base, ring_base, q, lane);
+    else if (px == 2) produce<TILE, SEGK, CW, MODE, IS_A, 2>(g, flags_base, ring_base, q, lane);
+    else produce<TILE, SEGK, CW, MODE, IS_A, 4>(g, flags_base, ring_base, q, lane);
+}
+
 // ---- consumer ----------------------------------------------------------------------------------------
 template <typename DT, int TILE, int SEGK, int CW, int MODE>
-__device__ void consume(const GemmArgs& g, uint32_t flags_base, uint32_t ring_base, int cw, int lane) {
+__device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, uint32_t ring_base, int cw, int lane) {
     constexpr int WTR = TILE / (CW / 2) / MFMA_M, WTC = TILE / 2 / MFMA_N;
     constexpr int CPR = SEGK / CHUNK_ELEMS;
     constexpr int RB = SEGK * 2;
@@ -362,19 +405,33 @@ __device__ void consume(const GemmArgs& g, uint32_t flags_base, uint32_t ring_ba
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) {
                     const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
-                    u32x4 a[WTR], b[WTC];
+                    // At most JB Bt fragments are resident; fragment j + JB replaces fragment j
+                    // right after its last use, so a 4 x 8 wave tile needs 32 fragment registers
+                    // next to its 128 accumulator registers.
+                    constexpr int JB = WTC > 4 ? 3 : WTC;
+                    u32x4 a[WTR], b[JB];
 #pragma unroll
                     for (int i = 0; i < WTR; ++i) a[i] = *(const CK_LDS u32x4*)(uintptr_t)(st + a_lane + coff + i * 16 * RB);
 #pragma unroll
-                    for (int j = 0; j < WTC; ++j) b[j] = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + j * 16 * RB);
-                    if (ks == KSTEPS - 1) {
+                    for (int j = 0; j < JB; ++j) b[j] = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + j * 16 * RB);
+                    if (ks == KSTEPS - 1 && JB == WTC) {
                         flag_add_after_reads(emptyA + fa_idx * 4);
                         flag_add(emptyB + fb_idx * 4);
                     }
 #pragma unroll
-                    for (int j = 0; j < WTC; ++j)
+                    for (int j = 0; j < WTC; ++j) {
+                        if (ks == KSTEPS - 1 && JB != WTC && j == WTC - 1) {
+                            flag_add_after_reads(emptyA + fa_idx * 4);
+                            flag_add(emptyB + fb_idx * 4);
+                        }
 #pragma unroll
-                        for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(b[j], a[i], acc[i][j]);
+                        for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(b[j % JB], a[i], acc[i][j]);
+                        if (j + JB < WTC) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            b[j % JB] = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + (j + JB) * 16 * RB);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
                 }
             } else {
                 // accumulator granularity: counters per (wave-tile row, 16-row block) and per
@@ -480,9 +537,9 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_pc_kernel(const GemmArgs g) {
 
     const uint32_t flags_base = lds0, ring_base = lds0 + fregion;
     if (wave < g.pa) {
-        produce<TILE, SEGK, CW, MODE, true>(g, flags_base, ring_base, wave, g.pa, lane);
+        produce_px<TILE, SEGK, CW, MODE, true>(g, flags_base, ring_base, wave, g.pa, lane);
     } else if (wave < g.pa + g.pb) {
-        produce<TILE, SEGK, CW, MODE, false>(g, flags_base, ring_base, wave - g.pa, g.pb, lane);
+        produce_px<TILE, SEGK, CW, MODE, false>(g, flags_base, ring_base, wave - g.pa, g.pb, lane);
     } else if (wave < g.pa + g.pb + CW) {
         consume<DT, TILE, SEGK, CW, MODE>(g, flags_base, ring_base, wave - g.pa - g.pb, lane);
     }
