@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fp16 GEMM M=N=K=8192 (fp32 accumulate/output) on one MI355X through the C ABI.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [tuning flags]
+
+A step is one launch of gemm_shmem_tc_async_opt_port over seeded synthetic A and Bt that are already
+resident in HBM. Prints ONE JSON line: whole-job TFLOP/s, the MFMA roofline of the kernel (flops per
+launch / average launch duration measured with HIP events on the launch stream, against the 2.5 PFLOP/s
+dense fp16 peak) and the CPU oracle timed on a bounded sample of the same workload.
+"""
+import argparse
+import importlib.util
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"mfma_f16": 2500.0, "valu_f32": 157.3}
+
+WORKLOADS = {
+    # name: (kind, dtype, M, N, K, distribution)
+    "config1_fp16_512": ("gemm", "f16", 512, 512, 512, "uniform"),
+    "config2_fp32_4096_simt": ("simt", "f32", 4096, 4096, 4096, "uniform"),
+    "config3_fp16_8192": ("gemm", "f16", 8192, 8192, 8192, "uniform"),
+    "config4_fp16_2048x2048x32768": ("gemm", "f16", 2048, 2048, 32768, "normal"),
+    "config5_bf16_6143x4097x3071": ("gemm", "bf16", 6143, 4097, 3071, "uniform"),
+}
+
+
+def load_package():
+    name = "ckopt_amd"
+    if name in sys.modules:
+        return sys.modules[name]
+    path = os.path.join(ROOT, "cuda-kernel-opt_amd", "__init__.py")
+    spec = importlib.util.spec_from_file_location(name, path, submodule_search_locations=[os.path.dirname(path)])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def cpu_baseline(ck, kind, dtype, a, b, M, N, K, budget_s=12.0):
+    """Times the CPU oracle on a bounded row sample of the same operands; returns the JSON object."""
+    from oracle import oracle as o
+    threads = o.lib().oracle_num_threads()
+
+    def run(rows):
+        t0 = time.perf_counter()
+        if kind == "gemm":
+            o.gemm(o.DT_F16 if dtype == "f16" else o.DT_BF16, a, b, rows=(0, rows), blocked=True)
+        else:
+            o.matmul(o.DT_F32, a, b, True, False, rows=(0, rows))
+        return time.perf_counter() - t0
+
+    rows = min(M, 16)
+    dt = run(rows)
+    while dt < budget_s / 4 and rows < M:
+        rows = min(M, max(rows * 2, int(rows * (budget_s / 2) / max(dt, 1e-3)) // 16 * 16))
+        dt = run(rows)
+    tflops = 2.0 * rows * N * K / dt * 1e-12
+    return {"value": round(tflops, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "first %d of %d rows of the same seeded operands (%.1f s), sequential-k fp32 loop of "
+                      "matmul_test.h:289-302 vectorised across output columns, %d OpenMP threads" % (rows, M, dt, threads)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="config3_fp16_8192", choices=sorted(WORKLOADS))
+    ap.add_argument("--tile", type=int, default=256)
+    ap.add_argument("--segk", type=int, default=64)
+    ap.add_argument("--stages", type=int, default=2)
+    ap.add_argument("--producers", type=int, default=2)
+    ap.add_argument("--consumers", type=int, default=8)
+    ap.add_argument("--group", type=int, default=4)
+    ap.add_argument("--mode", default="tile", choices=["tile", "wave", "acc"])
+    ap.add_argument("--bar-steps-a", type=int, default=0)
+    ap.add_argument("--bar-steps-b", type=int, default=0)
+    ap.add_argument("--cus", type=int, default=0, help="persistent grid size (default: all compute units)")
+    ap.add_argument("--block-rows", type=int, default=2, help="matmul_shmem: block_rows (SIMT workload only)")
+    ap.add_argument("--simt-tile", type=int, default=128)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every box of this build has one MI355X and the GEMM path has no "
+              "collective; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    if not torch.cuda.is_available():
+        print("no GPU visible: bench.py needs an MI355X", file=sys.stderr)
+        return 3
+    ck = load_package()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cus = args.cus or torch.cuda.get_device_properties(0).multi_processor_count
+
+    kind, dtype, M, N, K, dist = WORKLOADS[args.workload]
+    seed = 0xC0FFEE00 + int(args.workload[6])
+    ckdt = {"f16": ck.DT_F16, "bf16": ck.DT_BF16, "f32": ck.DT_F32}[dtype]
+    if dist == "uniform":
+        a = ck.fill_uniform(ckdt, (M, K), seed, 0, -1.0, 1.0)
+        b = ck.fill_uniform(ckdt, (N, K), seed, 1, -1.0, 1.0)
+    else:
+        a = ck.fill_normal(ckdt, (M, K), seed, 0, 0.0, 0.1)
+        b = ck.fill_normal(ckdt, (N, K), seed, 1, 0.0, 0.1)
+
+    def to_dev(x):
+        return torch.from_numpy(x.view(np.int16) if x.dtype == np.uint16 else x).to(dev)
+
+    da, db = to_dev(a), to_dev(b)
+    dd = torch.empty((M, N), dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream()
+
+    if kind == "gemm":
+        rows_a = rows_b = args.tile
+        if args.mode == "wave":
+            wtr = ck.get_warp_tile_rows(args.tile, args.consumers)
+            rows_a, rows_b = wtr * 16, ck.get_num_acc(args.tile, args.consumers) // wtr * 16
+        elif args.mode == "acc":
+            rows_a = rows_b = 16
+
+        def step():
+            ck.gemm_shmem_tc_async_opt_port(ckdt, da, db, None, dd, 1.0, 0.0, M, N, K, args.tile, args.segk,
+                                            args.bar_steps_a, args.bar_steps_b, rows_a, rows_b, args.group, args.stages,
+                                            args.producers, args.consumers, cus, stream)
+        peak, bound_name, arith = PEAK_TFLOPS["mfma_f16"], "mfma", dtype
+        kernel = "gemm_pc_kernel<%s, tile %d, seg_k %d, %dC+%dP waves, %s sync>" % (
+            dtype, args.tile, args.segk, args.consumers, args.producers, args.mode)
+    else:
+        def step():
+            ck.matmul_shmem(ck.DT_F32, da, db, dd, M, N, K, args.simt_tile, args.block_rows, True, stream)
+        peak, bound_name, arith = PEAK_TFLOPS["valu_f32"], "valu_f32", "f32"
+        kernel = "matmul_shmem_kernel<f32, tile %d, %d accumulators/thread>" % (args.simt_tile, args.simt_tile // args.block_rows)
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    if ck.device_status() != 0:
+        print("device status non-zero after warm-up: a bounded flag wait gave up", file=sys.stderr)
+        return 4
+
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for _ in range(args.steps):
+        step()
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kern_ms = ev0.elapsed_time(ev1) / args.steps   # HIP events on the launch stream; launches are back to back
+    if ck.device_status() != 0:
+        print("device status non-zero after the timed region", file=sys.stderr)
+        return 4
+
+    flops = 2.0 * M * N * K
+    value = flops / (wall_ms * 1e-3) * 1e-12
+    achieved = flops / (kern_ms * 1e-3) * 1e-12
+
+    # parity spot-check of what was just timed (oracle = checker, outside the timed region)
+    check = None
+    if not args.no_check:
+        from oracle import oracle as o
+        got = dd[:8].cpu().numpy()
+        if kind == "gemm":
+            ref = o.gemm(o.DT_F16 if dtype == "f16" else o.DT_BF16, a, b, rows=(0, 8))
+            nbad, worst = o.count_outside_rel(ref, got, 1e-2)
+        else:
+            ref = o.matmul(o.DT_F32, a, b, True, False, rows=(0, 8))
+            nbad, worst = o.count_outside_rel(ref, got, 1e-4)
+        check = {"rows_checked": 8, "outside_tolerance": nbad, "worst_ratio": round(worst, 8)}
+        if nbad:
+            print("parity check failed: %d elements outside tolerance" % nbad, file=sys.stderr)
+            return 5
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(args.workload)
+        except Exception:
+            traffic = None
+
+    out = {
+        "metric": "fp16_gemm_8192_tflops" if args.workload == "config3_fp16_8192" else args.workload + "_tflops",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": arith, "data": "synthetic",
+        "pct_of_peak": round(100.0 * value / peak, 2),
+        "config": {"workload": "%s: %s %dx%dx%d, A MxK and Bt NxK row-major, %s inputs from seed, fp32 accumulate/output"
+                               % (args.workload, dtype, M, N, K, "uniform[-1,1)" if dist == "uniform" else "N(0,1)*0.1"),
+                   "kernel": kernel, "tile_group_m": args.group, "num_stages": args.stages, "grid_cus": cus},
+        "roofline": {"bound": "mfma" if bound_name == "mfma" else "valu", "achieved": round(achieved, 2), "peak": peak,
+                     "unit": "TFLOP/s", "frac": round(achieved / peak, 4), "traffic": traffic,
+                     "kernel_ms": round(kern_ms, 5), "flops_per_launch": flops},
+    }
+    if check is not None:
+        out["parity_check"] = check
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(ck, kind, dtype, a, b, M, N, K)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,295 @@
+"""GPU parity tests of gemm_shmem_tc_async_opt_port (all through the C ABI) against the CPU oracle.
+
+Bars: bit-exact wherever the arithmetic is exact (constant matrices, small integers, identity,
+one-hot); |D - Dref| <= 1e-2 * (|Dref| + 1) for random fp16/bf16 inputs with fp32 accumulation, the
+tolerance BASELINE states. The three test kinds follow the reference's own drivers:
+constant-matrix correctness sweeps (port_2.cu:1171-1279), random accuracy counts (:1281-1391) and
+full-size runs checked through sampled rows and size-independent identities.
+"""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from tests import gpu_util as G
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-2  # |D - Dref| <= RTOL * (|Dref| + 1), fp16/bf16 inputs, fp32 accumulation
+
+
+def assert_close(oracle, ref, got, rtol=RTOL):
+    n, worst = oracle.count_outside_rel(ref, got, rtol)
+    assert n == 0, "%d elements outside tolerance, worst ratio %g" % (n, worst)
+
+
+def mode_rows(ck, t, mode):
+    if mode == "tile":
+        return t["tile_dim"], t["tile_dim"]
+    if mode == "wave":
+        return G.wave_mode_rows(ck, t)
+    return 16, 16
+
+
+def all_modes(ck, tile, cw):
+    """(mode, bar_steps_a, bar_steps_b) tuples legal for this tile / consumer count."""
+    wtr = ck.get_warp_tile_rows(tile, cw)
+    wtc = ck.get_num_acc(tile, cw) // wtr
+    out = [("tile", 0, 0)]
+    out += [("wave", sa, sb) for sa in range(cw // 2 + 1) for sb in range(3)]
+    out += [("acc", sa, sb) for sa in sorted({0, wtr // 2, wtr - 1}) for sb in sorted({0, wtc // 2, wtc - 1})]
+    return out
+
+
+def make_tuning(ck, tile, sk, stages, p, c, mode="tile", sa=0, sb=0, group=4, cus=256):
+    t = G.tuning(tile_dim=tile, segment_dim_k=sk, num_stages=stages, num_producer_warps=p, num_consumer_warps=c,
+                 bar_steps_a=sa, bar_steps_b=sb, tile_group_m=group, num_sms=cus)
+    t["bar_step_rows_a"], t["bar_step_rows_b"] = mode_rows(ck, t, mode)
+    return t
+
+
+def legal(ck, t):
+    return ck.check_gemm_tuning(t["tile_dim"], t["segment_dim_k"], t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"],
+                                t["bar_step_rows_b"], t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                t["num_consumer_warps"], t["num_sms"]) == ck.OK
+
+
+# ---- config 1: fp16 512^3, uniform[-1,1), seeded, checked against the full CPU reference -------------
+@pytest.mark.parametrize("tile,sk,stages,p,c", [(64, 64, 3, 2, 4), (128, 64, 2, 2, 4), (128, 64, 3, 4, 8),
+                                                 (128, 32, 4, 2, 8), (128, 128, 2, 8, 4), (256, 32, 4, 4, 8),
+                                                 (256, 64, 2, 2, 8)])
+def test_config1_fp16_512_uniform(ck, oracle, tile, sk, stages, p, c):
+    M = N = K = 512
+    a = ck.fill_uniform(ck.DT_F16, (M, K), 0xC0FFEE01, 0)
+    bt = ck.fill_uniform(ck.DT_F16, (N, K), 0xC0FFEE01, 1)
+    ref = oracle.gemm(oracle.DT_F16, a, bt)
+    d = G.run_gemm(ck, ck.DT_F16, a, bt, t=make_tuning(ck, tile, sk, stages, p, c))
+    assert_close(oracle, ref, d)
+    # the reference's accuracy criterion: count of |err| > 0.1 (matmul_test.h:320) must be zero too
+    assert oracle.count_incorrect(ref, d, 0.1) == 0
+
+
+# ---- constant matrices: the reference's correctness sweep, closed form alpha*1*10*K + beta*1 -------------
+def constant_sweep(ck):
+    tuples = []
+    for tile, c in ((64, 4), (64, 8), (128, 4), (128, 8), (256, 8)):
+        for sk in (32, 64, 128):
+            for (mode, sa, sb) in all_modes(ck, tile, c):
+                for stages, p, group in ((1, 2, 1), (3, 4, 3), (2, 8, 6)):
+                    t = make_tuning(ck, tile, sk, stages, p, c, mode, sa, sb, group)
+                    if legal(ck, t):
+                        tuples.append(t)
+    return tuples
+
+
+def test_constant_matrices_sweep(ck):
+    dim_max = 1024
+    a = G.to_dev(ck.fill_constant(ck.DT_F16, (dim_max * dim_max,), 1.0))
+    bt = G.to_dev(ck.fill_constant(ck.DT_F16, (dim_max * dim_max,), 10.0))
+    c = G.to_dev(ck.fill_constant(ck.DT_F32, (dim_max * dim_max,), 1.0))
+    d = torch.empty(dim_max * dim_max, dtype=torch.float32, device="cuda")
+    rng = np.random.default_rng(0xC0FFEE)
+    tuples = constant_sweep(ck)
+    assert len(tuples) > 150
+    # every 5th tuple at a random tile-multiple sub-dimension (reference: GetMatDim, matmul_test.h:263-268)
+    for idx, t in enumerate(tuples[::3]):
+        tile = t["tile_dim"]
+        dim = dim_max if idx % 5 else max(tile, int(rng.integers(0, dim_max + 1)) // tile * tile)
+        d.fill_(0)
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, a, bt, c, d, 1.0, 1.0, dim, dim, dim, t["tile_dim"], t["segment_dim_k"],
+                                        t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                        t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                        t["num_consumer_warps"], t["num_sms"])
+        assert ck.device_status() == 0, t
+        got = d[: dim * dim]
+        want = 10.0 * dim + 1.0
+        assert bool(torch.all(got == want)), (t, dim, float(got.min()), float(got.max()))
+        assert bool(torch.all(d[dim * dim:] == 0)), "wrote past the dim x dim result"
+
+
+# ---- small integers: exact for every summation order, so any race or misplaced fragment shows ----------
+@pytest.mark.parametrize("tile,c", [(64, 4), (64, 8), (128, 4), (128, 8), (256, 8)])
+def test_small_integers_bit_exact_all_sync_modes(ck, tile, c):
+    M, N, K = 2 * tile, 3 * tile, 640
+    a = ck.fill_int(ck.DT_F16, (M, K), 21, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 21, 1, -2, 2)
+    want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)
+    n = 0
+    for (mode, sa, sb), (sk, stages, p) in itertools.product(all_modes(ck, tile, c), ((32, 4, 2), (64, 2, 4), (128, 1, 2))):
+        t = make_tuning(ck, tile, sk, stages, p, c, mode, sa, sb, group=2)
+        if not legal(ck, t):
+            continue
+        d = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+        assert np.array_equal(d, want), (t, int((d != want).sum()))
+        n += 1
+    assert n >= 20
+
+
+def test_more_stages_than_segments_and_single_segment(ck):
+    # K / seg_k < num_stages: some stages are never filled
+    a = ck.fill_int(ck.DT_F16, (256, 128), 3, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (256, 128), 3, 1, -2, 2)
+    want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)
+    for sk, stages in ((128, 2), (64, 4), (32, 9)):
+        for mode, sa, sb in (("tile", 0, 0), ("wave", 1, 1), ("acc", 1, 2)):
+            d = G.run_gemm(ck, ck.DT_F16, a, bt, t=make_tuning(ck, 128, sk, stages, 2, 4, mode, sa, sb))
+            assert np.array_equal(d, want)
+
+
+def test_identity_and_one_hot(ck):
+    K = 256
+    a = ck.fill_uniform(ck.DT_F16, (384, K), 5, 0)
+    eye = np.eye(K, dtype=np.float16)
+    d = G.run_gemm(ck, ck.DT_F16, a, eye, t=make_tuning(ck, 128, 64, 2, 2, 4))
+    assert np.array_equal(d, a.astype(np.float32))
+    rng = np.random.default_rng(2)
+    perm = rng.permutation(K)
+    bt = np.zeros((K, K), dtype=np.float16)
+    bt[np.arange(K), perm] = 2.0
+    d = G.run_gemm(ck, ck.DT_F16, a, bt, t=make_tuning(ck, 64, 32, 3, 2, 8, "acc", 0, 1))
+    assert np.array_equal(d, 2.0 * a[:, perm].astype(np.float32))
+
+
+@pytest.mark.parametrize("alpha,beta", [(1.0, 1.0), (1.5, -0.75), (0.0, 2.0), (-2.0, 0.0)])
+def test_alpha_beta_textbook_form(ck, oracle, alpha, beta):
+    # D = alpha*A*Bt^T + beta*C as the CPU check states it (matmul_test.h:298), not alpha*(beta*C + A*Bt^T)
+    M, N, K = 384, 256, 512
+    a = ck.fill_uniform(ck.DT_F16, (M, K), 8, 0)
+    bt = ck.fill_uniform(ck.DT_F16, (N, K), 8, 1)
+    c = ck.fill_uniform(ck.DT_F32, (M, N), 8, 2)
+    ref = oracle.gemm(oracle.DT_F16, a, bt, c, alpha, beta)
+    for t in (make_tuning(ck, 128, 64, 2, 2, 4), make_tuning(ck, 256, 32, 4, 4, 8, "wave", 2, 1)):
+        d = G.run_gemm(ck, ck.DT_F16, a, bt, c, alpha, beta, t=t)
+        assert_close(oracle, ref, d)
+
+
+def test_bf16_uniform_and_exact(ck, oracle):
+    M, N, K = 512, 384, 768
+    a = ck.fill_uniform(ck.DT_BF16, (M, K), 9, 0)
+    bt = ck.fill_uniform(ck.DT_BF16, (N, K), 9, 1)
+    ref = oracle.gemm(oracle.DT_BF16, a, bt)
+    for t in (make_tuning(ck, 128, 64, 3, 4, 8), make_tuning(ck, 256, 64, 2, 2, 8), make_tuning(ck, 64, 128, 2, 2, 4, "acc", 1, 1)):
+        assert_close(oracle, ref, G.run_gemm(ck, ck.DT_BF16, a, bt, t=t))
+    ai = ck.fill_int(ck.DT_BF16, (M, K), 9, 2, -3, 3)
+    bi = ck.fill_int(ck.DT_BF16, (N, K), 9, 3, -3, 3)
+    want = (G.as_f64(True, ai) @ G.as_f64(True, bi).T).astype(np.float32)
+    assert np.array_equal(G.run_gemm(ck, ck.DT_BF16, ai, bi, t=make_tuning(ck, 128, 32, 4, 2, 8, "wave", 1, 2)), want)
+
+
+@pytest.mark.parametrize("M,N,K", [(200, 136, 104), (129, 257, 72), (1, 1, 8), (513, 64, 1000), (6143, 4097, 3072)])
+def test_ragged_edges_aligned_k(ck, oracle, M, N, K):
+    # M, N not multiples of the tile and K not a multiple of the segment: edges zero-filled / masked.
+    # The result lives in a larger allocation whose guard band must stay untouched.
+    a = ck.fill_int(ck.DT_F16, (M, K), 31, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 31, 1, -2, 2)
+    da, db = G.to_dev(a), G.to_dev(bt)
+    guard = 4096
+    buf = torch.full((M * N + 2 * guard,), -7.0, dtype=torch.float32, device="cuda")
+    d = buf[guard: guard + M * N]
+    big = M > 2000
+    for t in ([make_tuning(ck, 256, 64, 2, 4, 8)] if big else
+              [make_tuning(ck, 64, 32, 3, 2, 4), make_tuning(ck, 128, 64, 2, 2, 8, "wave", 1, 1),
+               make_tuning(ck, 256, 32, 4, 4, 8), make_tuning(ck, 128, 128, 1, 2, 4, "acc", 2, 2)]):
+        buf.fill_(-7.0)
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, da, db, None, d, 1.0, 0.0, M, N, K, t["tile_dim"], t["segment_dim_k"],
+                                        t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                        t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                        t["num_consumer_warps"], t["num_sms"])
+        assert ck.device_status() == 0
+        assert bool(torch.all(buf[:guard] == -7.0)) and bool(torch.all(buf[guard + M * N:] == -7.0))
+        got = d.cpu().numpy().reshape(M, N)
+        if big:
+            # exact integer identity instead of a full CPU product: row sums and column sums of D
+            ai, bi = a.astype(np.int64), bt.astype(np.int64)
+            assert np.array_equal(got.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
+            assert np.array_equal(got.astype(np.int64).sum(axis=0), bi @ ai.sum(axis=0))
+            rows = (0, 2000, M - 1)
+            for r in rows:
+                assert np.array_equal(got[r], (ai[r] @ bi.T).astype(np.float32))
+        else:
+            assert np.array_equal(got, (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32))
+
+
+def test_port_0_and_port_1_entry_points(ck):
+    M, N, K = 256, 384, 512
+    a = ck.fill_int(ck.DT_F16, (M, K), 41, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 41, 1, -2, 2)
+    want = torch.from_numpy((a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)).cuda()
+    da, db = G.to_dev(a), G.to_dev(bt)
+    d = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    ck.gemm_shmem_tc_async_opt_port_0(ck.DT_F16, da, db, None, d, 1.0, 0.0, M, N, K, 128, 64, 3, 2, 2, 4, 256)
+    assert ck.device_status() == 0 and bool(torch.equal(d, want))
+    for rows_a, rows_b in ((128, 128), (64, 64), (16, 16)):
+        d.zero_()
+        ck.gemm_shmem_tc_async_opt_port_1(ck.DT_F16, da, db, None, d, 1.0, 0.0, M, N, K, 128, 64, rows_a, rows_b, 3, 2, 4, 4, 256)
+        assert ck.device_status() == 0 and bool(torch.equal(d, want))
+
+
+def test_errors_with_device_pointers(ck):
+    a = torch.zeros(1 << 16, dtype=torch.float16, device="cuda")
+    d = torch.zeros(1 << 16, dtype=torch.float32, device="cuda")
+    t = G.tuning()
+    args = (t["tile_dim"], t["segment_dim_k"], t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+            t["tile_group_m"], t["num_stages"], t["num_producer_warps"], t["num_consumer_warps"], t["num_sms"])
+    with pytest.raises(ck.CkoptError) as e:  # LDS over budget is the launcher's check here, not the caller's
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, a, a, None, d, 1.0, 0.0, 128, 128, 128, 128, 128, 0, 0, 128, 128, 4, 3, 2, 4, 256)
+    assert e.value.code == ck.ERR_LDS_BUDGET
+    ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, a, a, None, d, 1.0, 0.0, 128, 128, 128, *args)
+    assert ck.device_status() == 0
+
+
+def test_launch_is_deterministic_and_swizzle_is_transparent(ck):
+    M = N = K = 1024
+    a = ck.fill_uniform(ck.DT_F16, (M, K), 77, 0)
+    bt = ck.fill_uniform(ck.DT_F16, (N, K), 77, 1)
+    t = make_tuning(ck, 256, 64, 2, 4, 8)
+    d1 = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+    d2 = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+    assert np.array_equal(d1.view(np.uint32), d2.view(np.uint32))
+    prev = ck.set_option(ck.OPT_SWIZZLE, 0)
+    try:
+        d3 = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+    finally:
+        ck.set_option(ck.OPT_SWIZZLE, prev)
+    assert np.array_equal(d1.view(np.uint32), d3.view(np.uint32))
+
+
+# ---- full-size configurations: sampled rows against the oracle + exact integer identities ----------------
+def full_size_check(ck, oracle, dtype, odt, M, N, K, t, fill, rows):
+    a, bt = fill(0, (M, K)), fill(1, (N, K))
+    d = G.run_gemm(ck, dtype, a, bt, t=t)
+    for r0 in rows:
+        ref = oracle.gemm(odt, a, bt, rows=(r0, r0 + 8))
+        assert_close(oracle, ref, d[r0:r0 + 8])
+    assert np.isfinite(d).all()
+    # linearity checksum in float64: D @ 1 == A @ (Bt^T @ 1)
+    bis16 = dtype == ck.DT_BF16
+    lhs = d.astype(np.float64).sum(axis=1)
+    rhs = G.as_f64(bis16, a) @ G.as_f64(bis16, bt).sum(axis=0)
+    scale = (np.abs(G.as_f64(bis16, a)) @ np.abs(G.as_f64(bis16, bt)).sum(axis=0)) + 1.0
+    assert np.max(np.abs(lhs - rhs) / scale) < 1e-4
+
+
+def test_config3_fp16_8192_headline(ck, oracle):
+    M = N = K = 8192
+    t = make_tuning(ck, 256, 64, 2, 2, 8)
+    full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t,
+                    lambda s, shape: ck.fill_uniform(ck.DT_F16, shape, 0xC0FFEE03, s), rows=(0, 4000, 8184))
+    # exact: small integers at full size
+    a = ck.fill_int(ck.DT_F16, (M, K), 0xC0FFEE03, 2, -1, 1)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 0xC0FFEE03, 3, -1, 1)
+    d = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+    ai, bi = a.astype(np.int64), bt.astype(np.int64)
+    assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
+    assert np.array_equal(d.astype(np.int64).sum(axis=0), bi @ ai.sum(axis=0))
+    assert np.array_equal(d[4095], (ai[4095] @ bi.T).astype(np.float32))
+
+
+def test_config4_long_k_shift_sync_regime(ck, oracle):
+    M = N = 2048
+    K = 32768
+    fill = lambda s, shape: ck.fill_normal(ck.DT_F16, shape, 0xC0FFEE04, s, 0.0, 0.1)
+    for t in (make_tuning(ck, 128, 64, 4, 4, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 4, 2),
+              make_tuning(ck, 128, 64, 4, 4, 8, "acc", 1, 3)):
+        full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t, fill, rows=(0, 1024))

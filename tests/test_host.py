@@ -1,0 +1,193 @@
+"""CPU-only tests of the host side: the C ABI loads and exports what include/ckopt.h declares,
+parameter legality mirrors the reference launcher's asserts, the index helpers agree with the oracle's
+restatement of the reference on the reference's domain, and the seeded generator is reproducible.
+No kernel is launched here.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ckopt.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ckopt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(ck):
+    lib = ctypes.CDLL(ck.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 18
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(ck.EXPORTED_SYMBOLS) == names
+
+
+def test_num_acc_and_warp_tile_rows_match_reference_closed_forms(ck, oracle):
+    L = oracle.lib()
+    for t in (64, 128):
+        for c in (4, 8):
+            assert ck.get_num_acc(t, c) == L.oracle_get_num_acc(t, c)
+            assert ck.get_warp_tile_rows(t, c) == L.oracle_get_warp_tile_rows(t, c)
+    # extension to 256: (C/2) x 2 wave tiles of 16x16 blocks
+    assert ck.get_num_acc(256, 8) == 32 and ck.get_warp_tile_rows(256, 8) == 4
+    with pytest.raises(ck.CkoptError):
+        ck.get_num_acc(96, 4)
+
+
+@pytest.mark.parametrize("M,N,t,g", [(512, 512, 128, 1), (1024, 768, 128, 3), (640, 1280, 64, 4), (256, 256, 64, 6),
+                                     (2048, 2048, 256, 4)])
+def test_tile_offset_matches_reference_order(ck, oracle, M, N, t, g):
+    L = oracle.lib()
+    for tc in range((M // t) * (N // t)):
+        assert ck.get_tile_offset_cd(M, N, t, g, tc) == L.oracle_get_tile_offset_cd(M, N, t, g, tc)
+
+
+def test_tile_offset_ragged_is_a_bijection_and_64_bit(ck):
+    M, N, t, g = 6143, 4097, 128, 5
+    tm, tn = -(-M // t), -(-N // t)
+    got = sorted(ck.get_tile_offset_cd(M, N, t, g, tc) for tc in range(tm * tn))
+    assert got == sorted(r * t * N + c * t for r in range(tm) for c in range(tn))
+    # past int32: 65536 x 65536, last tile
+    big = ck.get_tile_offset_cd(65536, 65536, 256, 4, 256 * 256 - 1)
+    assert big == (65536 - 256) * 65536 + (65536 - 256)
+
+
+def test_lds_req_layout(ck):
+    # flag region rounded to 1 KiB + stages x 2 operands x tile x seg_k x 2 bytes, no padding
+    assert ck.get_lds_req(128, 64, 0, 0, 128, 128, 2, 4) == 1024 + 2 * 2 * 128 * 64 * 2
+    assert ck.get_lds_req(256, 32, 0, 0, 256, 256, 4, 8) == 1024 + 4 * 2 * 256 * 32 * 2
+    # wave mode: 2*(sa+1) + 2*(sb+1) counters per stage; acc mode: 2*(C/2)*(sa+1) + 2*2*(sb+1)
+    assert ck.get_lds_req(128, 64, 2, 2, 64, 64, 3, 4) == 1024 + 3 * 2 * 128 * 64 * 2
+    assert ck.get_lds_req(256, 32, 3, 7, 16, 16, 16, 8) == 4096 + 16 * 2 * 256 * 32 * 2
+    with pytest.raises(ck.CkoptError):
+        ck.get_lds_req(128, 64, 0, 0, 48, 48, 2, 4)  # not one of the three granularities
+
+
+def tup(**kw):
+    d = dict(tile_dim=128, segment_dim_k=64, bar_steps_a=0, bar_steps_b=0, bar_step_rows_a=128, bar_step_rows_b=128,
+             tile_group_m=4, num_stages=2, num_producer_waves=2, num_consumer_waves=4, num_cus=256)
+    d.update(kw)
+    return d
+
+
+def test_tuning_legality_mirrors_reference_asserts(ck):
+    ok = lambda **kw: ck.check_gemm_tuning(**tup(**kw))
+    assert ok() == ck.OK
+    assert ok(tile_dim=96, bar_step_rows_a=96, bar_step_rows_b=96) == ck.ERR_BAD_PARAM     # port_2.cu:1112
+    assert ok(segment_dim_k=48) == ck.ERR_BAD_PARAM                                          # :1113
+    assert ok(num_producer_waves=3) == ck.ERR_BAD_PARAM                                      # :1122
+    assert ok(num_consumer_waves=6) == ck.ERR_BAD_PARAM                                      # :1123
+    assert ok(num_stages=0) == ck.ERR_BAD_PARAM                                              # :1121
+    assert ok(tile_group_m=0) == ck.ERR_BAD_PARAM
+    # barrier-mode triple (:1116-1120): wave-tile mode t=128, C=4 -> rows 64, cols 64, steps <= 2 / <= 2
+    assert ok(bar_step_rows_a=64, bar_step_rows_b=64, bar_steps_a=2, bar_steps_b=2) == ck.OK
+    assert ok(bar_step_rows_a=64, bar_step_rows_b=64, bar_steps_a=3, bar_steps_b=2) == ck.ERR_BAD_PARAM
+    assert ok(bar_step_rows_a=64, bar_step_rows_b=32) == ck.ERR_BAD_PARAM
+    # accumulator mode: steps strictly below wave tile rows / cols (4 x 4 for t=128, C=4)
+    assert ok(bar_step_rows_a=16, bar_step_rows_b=16, bar_steps_a=3, bar_steps_b=3) == ck.OK
+    assert ok(bar_step_rows_a=16, bar_step_rows_b=16, bar_steps_a=4, bar_steps_b=0) == ck.ERR_BAD_PARAM
+    # LDS budget: 160 KiB
+    assert ok(num_stages=4) == ck.OK                                   # 1 KiB + 128 KiB
+    assert ok(num_stages=5) == ck.ERR_LDS_BUDGET
+    assert ok(tile_dim=256, bar_step_rows_a=256, bar_step_rows_b=256, num_consumer_waves=8, segment_dim_k=64, num_stages=3) == ck.ERR_LDS_BUDGET
+    # register budget: a 256 tile with 4 consumer waves needs 256 accumulator registers per wave;
+    # 8 producers + 8 consumers at tile 256 exceed the instance's wave count (the reference's own
+    # P=8, C=8 launch failure, port_1.cu:35-42, becomes an error code)
+    assert ok(tile_dim=256, bar_step_rows_a=256, bar_step_rows_b=256, num_consumer_waves=4) == ck.ERR_NO_INSTANCE
+    assert ok(tile_dim=256, bar_step_rows_a=256, bar_step_rows_b=256, num_consumer_waves=8, num_producer_waves=8,
+              segment_dim_k=32) == ck.ERR_NO_INSTANCE
+    assert ok(tile_dim=256, bar_step_rows_a=256, bar_step_rows_b=256, num_consumer_waves=8, num_producer_waves=4,
+              segment_dim_k=32, num_stages=4) == ck.OK
+
+
+def test_launch_rejects_bad_arguments_before_touching_the_gpu(ck):
+    # null pointers and illegal shapes are reported without any HIP call
+    args = dict(tile_dim=128, segment_dim_k=64, bar_steps_a=0, bar_steps_b=0, bar_step_rows_a=128, bar_step_rows_b=128,
+                tile_group_m=4, num_stages=2, num_producer_warps=2, num_consumer_warps=4, num_sms=256)
+    with pytest.raises(ck.CkoptError) as e:
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, None, None, None, None, 1.0, 0.0, 256, 256, 256, **args)
+    assert e.value.code == ck.ERR_NULL
+    with pytest.raises(ck.CkoptError) as e:
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F32, 16, 16, None, 16, 1.0, 0.0, 256, 256, 256, **args)
+    assert e.value.code == ck.ERR_BAD_PARAM
+    with pytest.raises(ck.CkoptError) as e:
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, 16, 16, None, 16, 1.0, 0.0, 0, 256, 256, **args)
+    assert e.value.code == ck.ERR_BAD_PARAM
+    with pytest.raises(ck.CkoptError) as e:  # beta != 0 needs C
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, 16, 16, None, 16, 1.0, 1.0, 256, 256, 256, **args)
+    assert e.value.code == ck.ERR_NULL
+    with pytest.raises(ck.CkoptError) as e:  # misaligned A
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, 18, 16, None, 16, 1.0, 0.0, 256, 256, 256, **args)
+    assert e.value.code == ck.ERR_ALIGNMENT
+
+
+def test_matmul_shmem_tuning_legality(ck):
+    # reference: tile % block_rows == 0, accumulators per thread bounded, tile*block_rows <= max threads
+    # (matmul_shmem.cu:153-155, :198-206)
+    assert ck.check_matmul_shmem_tuning(32, 8) == ck.OK
+    assert ck.check_matmul_shmem_tuning(128, 2) == ck.OK       # 64 accumulators per thread (extension)
+    assert ck.check_matmul_shmem_tuning(128, 4) == ck.OK
+    assert ck.check_matmul_shmem_tuning(128, 16) == ck.ERR_NO_INSTANCE   # 2048 threads
+    assert ck.check_matmul_shmem_tuning(64, 3) == ck.ERR_BAD_PARAM
+    assert ck.check_matmul_shmem_tuning(48, 4) == ck.ERR_BAD_PARAM
+    assert ck.check_matmul_shmem_tuning(32, 1) == ck.ERR_NO_INSTANCE     # 32 threads: less than a wavefront
+    assert ck.matmul_shmem_lds_req(ck.DT_F32, 128) == 2 * 2 * 16 * 132 * 4
+    with pytest.raises(ck.CkoptError) as e:
+        ck.matmul_shmem(ck.DT_F32, 16, 16, 16, 100, 128, 128, 32, 8)
+    assert e.value.code == ck.ERR_BAD_PARAM
+
+
+def test_splitmix64_known_answers(oracle):
+    # first outputs of SplitMix64 seeded with 1234567 (Vigna's reference implementation)
+    z = oracle.splitmix64_at(1234567, np.arange(5))
+    assert [int(v) for v in z] == [6457827717110365317, 3203168211198807973, 9817491932198370423,
+                                   4593380528125082431, 16408922859458223821]
+
+
+def test_uniform_generator_matches_numpy_restatement_and_is_seeded(ck, oracle):
+    n = 10000
+    for seed, stream in ((0xC0FFEE01, 0), (0xC0FFEE01, 1), (42, 7)):
+        f32 = ck.fill_uniform(ck.DT_F32, (n,), seed, stream, -1.0, 1.0)
+        want = oracle.uniform_f32(n, seed, stream, -1.0, 1.0)
+        assert np.array_equal(f32, want)
+        f16 = ck.fill_uniform(ck.DT_F16, (n,), seed, stream, -1.0, 1.0)
+        assert np.array_equal(f16.view(np.uint16), want.astype(np.float16).view(np.uint16))   # RNE to half
+        b16 = ck.fill_uniform(ck.DT_BF16, (n,), seed, stream, -1.0, 1.0)
+        tb = torch.from_numpy(want).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(b16, tb)                                                          # RNE to bf16
+    a = ck.fill_uniform(ck.DT_F32, (n,), 1, 0)
+    assert np.array_equal(a, ck.fill_uniform(ck.DT_F32, (n,), 1, 0))
+    assert not np.array_equal(a, ck.fill_uniform(ck.DT_F32, (n,), 2, 0))
+    assert not np.array_equal(a, ck.fill_uniform(ck.DT_F32, (n,), 1, 1))
+    assert a.min() >= -1.0 and a.max() < 1.0 and abs(float(a.mean())) < 0.03
+    # a sub-range reproduces the same values: element i depends on (seed, stream, i) only
+    assert np.array_equal(ck.fill_uniform(ck.DT_F32, (100,), 1, 0), a[:100])
+
+
+def test_half_rounding_edge_cases(ck):
+    vals = np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 6e-8, 2.98e-8, 2.99e-8, 6.1e-5, 1.0009765625, 1.00048828125,
+                     -3.14159, 1e6, -1e6], dtype=np.float32)
+    for v in vals:
+        got = ck.fill_constant(ck.DT_F16, (1,), float(v)).view(np.uint16)[0]
+        with np.errstate(over="ignore"):
+            want = np.float32(v).astype(np.float16).view(np.uint16)
+        assert got == want, (v, hex(got), hex(want))
+
+
+def test_normal_and_int_generators(ck):
+    x = ck.fill_normal(ck.DT_F32, (200000,), 5, 0, 0.0, 0.1)
+    assert abs(float(x.mean())) < 2e-3 and abs(float(x.std()) - 0.1) < 2e-3
+    assert np.array_equal(x, ck.fill_normal(ck.DT_F32, (200000,), 5, 0, 0.0, 0.1))
+    k = ck.fill_int(ck.DT_I32, (50000,), 9, 3, -10, 10)
+    assert k.min() == -10 and k.max() == 10 and len(np.unique(k)) == 21
+    h = ck.fill_int(ck.DT_F16, (1000,), 9, 3, -2, 2)
+    assert set(np.unique(h.astype(np.int32))) == {-2, -1, 0, 1, 2}
+    c = ck.fill_constant(ck.DT_BF16, (8,), 10.0)
+    assert np.all(c == 0x4120)
