@@ -12,7 +12,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libckopt.so")
+# CKOPT_LIB selects another build of the same library (e.g. a measurement variant)
+LIB_PATH = os.environ.get("CKOPT_LIB") or os.path.join(HERE, "lib", "libckopt.so")
 
 DT_F16, DT_BF16, DT_F32, DT_I32 = 0, 1, 2, 3
 OK, ERR_BAD_PARAM, ERR_LDS_BUDGET, ERR_NO_INSTANCE, ERR_HIP, ERR_ALIGNMENT, ERR_NULL, ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6, -7
@@ -49,6 +50,10 @@ _lib.ckopt_check_matmul_shmem_tuning.restype = _i
 _lib.ckopt_check_matmul_shmem_tuning.argtypes = [_i, _i]
 _lib.ckopt_device_status.restype = _i
 _lib.ckopt_device_status.argtypes = [_p]
+_lib.ckopt_last_launch_clocks.restype = _i
+_lib.ckopt_last_launch_clocks.argtypes = [_p, ctypes.POINTER(_u64), ctypes.POINTER(_u64)]
+_lib.ckopt_probe_counters.restype = _i
+_lib.ckopt_probe_counters.argtypes = [_p, ctypes.POINTER(ctypes.c_uint), _i]
 _lib.ckopt_set_option.restype = _i
 _lib.ckopt_set_option.argtypes = [_i, _i]
 _lib.ckopt_fill_uniform.restype = _i
@@ -66,7 +71,8 @@ EXPORTED_SYMBOLS = [
     "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_1",
     "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
-    "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_set_option", "ckopt_fill_uniform",
+    "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks", "ckopt_probe_counters",
+    "ckopt_set_option", "ckopt_fill_uniform",
     "ckopt_fill_normal", "ckopt_fill_int", "ckopt_fill_constant", "ckopt_error_string",
 ]
 
@@ -191,6 +197,20 @@ def device_status(stream=None):
     if r < 0:
         raise CkoptError(r, "device_status")
     return r
+
+
+def last_launch_clocks(stream=None):
+    """(shader cycles, 100 MHz reference ticks) workgroup 0 of the last GEMM launch ran for."""
+    c, w = _u64(0), _u64(0)
+    _check(_lib.ckopt_last_launch_clocks(_stream(stream), ctypes.byref(c), ctypes.byref(w)), "last_launch_clocks")
+    return int(c.value), int(w.value)
+
+
+def probe_counters(nwaves=16, stream=None):
+    """Per-wave counters of a measurement build (zeros otherwise): list of 8-word lists."""
+    buf = (ctypes.c_uint * (nwaves * 8))()
+    _check(_lib.ckopt_probe_counters(_stream(stream), buf, nwaves * 8), "probe_counters")
+    return [list(buf[w * 8:(w + 1) * 8]) for w in range(nwaves)]
 
 
 def set_option(key, value):

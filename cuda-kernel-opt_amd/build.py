@@ -43,11 +43,11 @@ def headers_mtime():
     return m
 
 
-def compile_one(src, force):
-    obj = os.path.join(BUILD, os.path.basename(src) + ".o")
+def compile_one(src, force, build_dir=None, extra=()):
+    obj = os.path.join(build_dir or BUILD, os.path.basename(src) + ".o")
     if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), headers_mtime()):
         return obj, "up to date"
-    flags = DEVICE_FLAGS if src.endswith(".hip") else HOST_FLAGS
+    flags = (DEVICE_FLAGS if src.endswith(".hip") else HOST_FLAGS) + list(extra)
     cmd = [HIPCC] + flags + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -55,29 +55,35 @@ def compile_one(src, force):
     return obj, "compiled"
 
 
-def build(jobs=8, force=False, verbose=True):
-    os.makedirs(BUILD, exist_ok=True)
-    os.makedirs(LIBDIR, exist_ok=True)
+def build(jobs=8, force=False, verbose=True, out_dir=None, extra=()):
+    """out_dir/extra: build a variant (extra compiler flags, e.g. -DCK_PROBE_NO_MFMA) into another directory."""
+    build_dir = os.path.join(out_dir, "build") if out_dir else BUILD
+    lib_dir = out_dir if out_dir else LIBDIR
+    lib = os.path.join(lib_dir, "libckopt.so")
+    os.makedirs(build_dir, exist_ok=True)
+    os.makedirs(lib_dir, exist_ok=True)
     srcs = sources()
     objs = []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        for obj, what in ex.map(lambda s: compile_one(s, force), srcs):
+        for obj, what in ex.map(lambda s: compile_one(s, force, build_dir, extra), srcs):
             if verbose:
                 print("[build] %-40s %s" % (os.path.basename(obj), what), flush=True)
             objs.append(obj)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed: %s\n%s\n%s" % (" ".join(cmd), r.stdout, r.stderr))
     if verbose:
-        print("[build] linked %s" % LIB, flush=True)
-    return LIB
+        print("[build] linked %s" % lib, flush=True)
+    return lib
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--out-dir", default=None)
+    ap.add_argument("--define", action="append", default=[])
     a = ap.parse_args()
-    build(a.jobs, a.force)
+    build(a.jobs, a.force, out_dir=a.out_dir, extra=["-D" + d for d in a.define])
     sys.exit(0)

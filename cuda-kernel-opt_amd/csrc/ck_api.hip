@@ -19,7 +19,7 @@ hipError_t launch_matmul_shmem(int dtype, int tile, int accs, bool bt, dim3 grid
 }  // namespace ck
 
 // One status word per device; the kernels OR a bit into it when a bounded flag wait gives up.
-__device__ unsigned int ck_status_word = 0;
+__device__ unsigned int ck_status_word[8 + 16 * 8] = {};  // [8..]: per-wave cycle counters of measurement builds
 
 namespace {
 
@@ -219,6 +219,34 @@ int ckopt_device_status(void* stream) {
         if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
     }
     return (int)(v & 0x7fffffffu);
+}
+
+int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* ref_ticks) {
+    unsigned int* p = nullptr;
+    const int rc = status_ptr_for_current_device(&p);
+    if (rc != ck::CK_OK) return rc;
+    if (!shader_cycles || !ref_ticks) return ck::CK_ERR_NULL;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned int v[8] = {};
+    if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
+    if (hipMemcpyAsync(v, p, sizeof(v), hipMemcpyDeviceToHost, s) != hipSuccess) return ck::CK_ERR_HIP;
+    if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
+    *shader_cycles = (uint64_t)v[2] | ((uint64_t)v[3] << 32);
+    *ref_ticks = (uint64_t)v[4] | ((uint64_t)v[5] << 32);
+    return ck::CK_OK;
+}
+
+int ckopt_probe_counters(void* stream, unsigned int* out, int nwords) {
+    unsigned int* p = nullptr;
+    const int rc = status_ptr_for_current_device(&p);
+    if (rc != ck::CK_OK) return rc;
+    if (!out) return ck::CK_ERR_NULL;
+    if (nwords < 0 || nwords > 16 * 8) return ck::CK_ERR_BAD_PARAM;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
+    if (hipMemcpyAsync(out, p + 8, sizeof(unsigned int) * nwords, hipMemcpyDeviceToHost, s) != hipSuccess) return ck::CK_ERR_HIP;
+    if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
+    return ck::CK_OK;
 }
 
 int ckopt_set_option(int key, int value) {

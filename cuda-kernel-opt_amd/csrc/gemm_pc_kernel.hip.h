@@ -42,6 +42,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define CK_LDS __attribute__((address_space(3)))
 
+// Bt fragments kept resident per k-step when a wave tile has more than four block columns
+#ifndef CK_RESIDENT_BT_FRAGS
+#define CK_RESIDENT_BT_FRAGS 3
+#endif
+
 struct GemmArgs {
     const void* A;
     const void* Bt;
@@ -58,7 +63,8 @@ struct GemmArgs {
     int num_xcd;
     int vec_store;  // D (and C) 16-byte aligned with N % 4 == 0
     uint32_t spin_limit;
-    unsigned int* status;  // device word: OR of CK_STATUS_* bits
+    unsigned int* status;  // device words: [0] OR of CK_STATUS_* bits, [2..3] shader cycles and [4..5] 100 MHz
+                           // ticks workgroup 0 spent in the last launch (actual-clock evidence)
 };
 
 enum : unsigned { CK_STATUS_PRODUCER_TIMEOUT = 1u, CK_STATUS_CONSUMER_TIMEOUT = 2u };
@@ -123,11 +129,19 @@ struct Spin {
     unsigned int* status;
     unsigned bit;
     bool dead;
+#if defined(CK_PROBE_TIMING)  // measurement build only: cycles spent and calls made in flag waits
+    unsigned long long wait_cycles = 0;
+    unsigned wait_calls = 0, wait_polls = 0;
+#endif
 };
 __device__ __forceinline__ bool flag_ready(uint32_t addr, uint32_t target) { return (int32_t)(flag_load(addr) - target) >= 0; }
 __device__ __forceinline__ void wait_flag_ge(uint32_t addr, uint32_t target, Spin& sp) {
     if (sp.dead) return;
     uint32_t n = 0;
+#if defined(CK_PROBE_TIMING)
+    const unsigned long long t0 = clock64();
+    struct Acc { Spin& s; unsigned long long t0; uint32_t& n; __device__ ~Acc() { s.wait_cycles += clock64() - t0; s.wait_calls++; s.wait_polls += n; } } acc_{sp, t0, n};
+#endif
     while (!flag_ready(addr, target)) {
         if (++n > sp.limit) {
             sp.dead = true;
@@ -189,6 +203,10 @@ template <int DEPTH>
 __device__ __forceinline__ void producer_wait(uint32_t addr, uint32_t target, SignalQueue<DEPTH>& q, Spin& sp) {
     if (target == 0 || sp.dead) return;
     uint32_t n = 0;
+#if defined(CK_PROBE_TIMING)
+    const unsigned long long t0 = clock64();
+    struct Acc { Spin& s; unsigned long long t0; uint32_t& n; __device__ ~Acc() { s.wait_cycles += clock64() - t0; s.wait_calls++; s.wait_polls += n; } } acc_{sp, t0, n};
+#endif
     while (!flag_ready(addr, target)) {
         if (q.pending()) {
             q.pop_front();
@@ -256,6 +274,9 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
     const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
     const int64_t total_tiles = (int64_t)g.tiles_m * g.tiles_n;
 
+#if defined(CK_PROBE_NO_SYNC)  // measurement build only: consumers run without any flag traffic
+    return;
+#endif
     Spin sp{g.spin_limit, g.status, CK_STATUS_PRODUCER_TIMEOUT, false};
     SignalQueue<MODE == CK_SYNC_TILE ? 3 : MODE == CK_SYNC_WAVE ? 4 : 8> sq;
     sq.init();
@@ -303,6 +324,10 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
                     if (sub <= s_own) producer_wait(fl + (empty_off + unit * (s_own + 1) + sub) * 4, readers * fill, sq, sp);
                 }
                 // ---- this wave's share of the row block, straight into LDS
+#if defined(CK_PROBE_NO_LOADS)  // measurement build only: producers signal without loading
+                if (true) {
+                } else
+#endif
                 if (fast) {
                     const uint32_t soff0 = (uint32_t)k0 * 2u;
 #pragma unroll
@@ -343,6 +368,12 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
         }
     }
     sq.drain();
+#if defined(CK_PROBE_TIMING)
+    if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
+        unsigned* o = g.status + 8 + (threadIdx.x >> 6) * 8;
+        o[0] = (unsigned)sp.wait_cycles; o[1] = (unsigned)(sp.wait_cycles >> 32); o[2] = sp.wait_calls; o[3] = sp.wait_polls;
+    }
+#endif
 }
 
 template <int TILE, int SEGK, int CW, int MODE, bool IS_A>
@@ -371,14 +402,19 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
     // lane -> fragment element: row (lane % 16) of a 16-row block, logical chunk kstep*4 + lane/16
     const int lr = lane & 15, lg = lane >> 4;
     const int key = g.swizzle ? swizzle_key(lr, CPR) : 0;  // same for every 16-row block
-    const uint32_t a_lane = (uint32_t)(R * WTR * 16 + lr) * RB;
-    const uint32_t b_lane = (uint32_t)OPB + (uint32_t)(Cc * WTC * 16 + lr) * RB;
+    // Per-lane LDS offset of the k-step-0 fragment chunk. Row offsets are multiples of the row size
+    // and stage bases multiples of 1 KiB, so the chunk of k-step ks is reached by XOR with ks * 64:
+    // ((ks*4 + lg) ^ key) * 16 == ((lg ^ key) * 16) ^ (ks * 64).
+    const uint32_t a_lane = (uint32_t)(R * WTR * 16 + lr) * RB + (uint32_t)((lg ^ key) * CHUNK_BYTES);
+    const uint32_t b_lane = (uint32_t)OPB + (uint32_t)(Cc * WTC * 16 + lr) * RB + (uint32_t)((lg ^ key) * CHUNK_BYTES);
 
     const int grid = gridDim.x;
     const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
     const int64_t total_tiles = (int64_t)g.tiles_m * g.tiles_n;
     Spin sp{g.spin_limit, g.status, CK_STATUS_CONSUMER_TIMEOUT, false};
 
+    // waves are dealt to the four SIMDs round-robin, so consumer cw shares its SIMD with cw +- 4
+    const bool burst_hi = (cw & 4) == 0;
     // WAVE mode: which counters this wave uses
     const bool individual = (MODE == CK_SYNC_WAVE) && R < sa && Cc < sb;
     int fa_idx = 0, fb_idx = 0;
@@ -386,6 +422,10 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
 
     int stage = 0;
     uint32_t fill = 0;
+    uint32_t pre_a = 0, pre_b = 0;  // "full" counters of the upcoming segment, read ahead of time
+#if defined(CK_PROBE_TIMING)
+    unsigned prefetch_hits = 0;
+#endif
     for (int64_t tc = slot; tc < total_tiles; tc += grid) {
         const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
         f32x4 acc[WTR][WTC];
@@ -400,36 +440,87 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
             const uint32_t fullA = fl, emptyA = fl + ua * 4, fullB = fl + 2 * ua * 4, emptyB = fl + (2 * ua + ub) * 4;
 
             if (MODE != CK_SYNC_ACC) {
-                wait_flag_ge(fullA + fa_idx * 4, pa * (fill + 1), sp);
-                wait_flag_ge(fullB + fb_idx * 4, pb * (fill + 1), sp);
+                // The two "full" counters of this segment were read one segment ahead (behind the
+                // previous segment's fragment reads); poll only if they were not there yet.
+#if !defined(CK_PROBE_NO_SYNC)
+                const uint32_t seen_a = __builtin_amdgcn_readfirstlane(pre_a);
+                const uint32_t seen_b = __builtin_amdgcn_readfirstlane(pre_b);
+                if ((int32_t)(seen_a - pa * (fill + 1)) < 0) wait_flag_ge(fullA + fa_idx * 4, pa * (fill + 1), sp);
+                if ((int32_t)(seen_b - pb * (fill + 1)) < 0) wait_flag_ge(fullB + fb_idx * 4, pb * (fill + 1), sp);
+#if defined(CK_PROBE_TIMING)
+                if ((int32_t)(seen_a - pa * (fill + 1)) >= 0 && (int32_t)(seen_b - pb * (fill + 1)) >= 0) prefetch_hits++;
+#endif
+                asm volatile("" ::: "memory");
+                {
+                    const int nstage = stage + 1 == S ? 0 : stage + 1;
+                    const uint32_t nfl = flags_base + (uint32_t)nstage * fps * 4;
+                    pre_a = *(volatile CK_LDS uint32_t*)(uintptr_t)(nfl + fa_idx * 4);
+                    pre_b = *(volatile CK_LDS uint32_t*)(uintptr_t)(nfl + 2 * ua * 4 + fb_idx * 4);
+                }
+#endif
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) {
-                    const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
+                    const uint32_t pa_k = (st + a_lane) ^ (uint32_t)(ks * 64), pb_k = (st + b_lane) ^ (uint32_t)(ks * 64);
                     // At most JB Bt fragments are resident; fragment j + JB replaces fragment j
                     // right after its last use, so a 4 x 8 wave tile needs 32 fragment registers
                     // next to its 128 accumulator registers.
-                    constexpr int JB = WTC > 4 ? 3 : WTC;
+                    constexpr int JB = WTC > 4 ? CK_RESIDENT_BT_FRAGS : WTC;
                     u32x4 a[WTR], b[JB];
+                    // Fragment-load phase at low priority, MFMA burst at a raised one. The two consumer
+                    // waves that share a SIMD raise to DIFFERENT levels: when both have MFMAs ready one
+                    // of them wins the matrix core outright, finishes its burst first and loads its next
+                    // fragments while the other bursts, so the pair settles into ping-pong instead of
+                    // stalling on LDS latency in lockstep.
+                    __builtin_amdgcn_s_setprio(0);
+#if defined(CK_PROBE_NO_LDS)  // measurement build only: fragments are made up in registers
 #pragma unroll
-                    for (int i = 0; i < WTR; ++i) a[i] = *(const CK_LDS u32x4*)(uintptr_t)(st + a_lane + coff + i * 16 * RB);
+                    for (int i = 0; i < WTR; ++i) a[i] = u32x4{pa_k, pa_k + i, 1u, 2u};
 #pragma unroll
-                    for (int j = 0; j < JB; ++j) b[j] = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + j * 16 * RB);
+                    for (int j = 0; j < JB; ++j) b[j] = u32x4{pb_k, pb_k + j, 3u, 4u};
+#else
+#pragma unroll
+                    for (int i = 0; i < WTR; ++i) a[i] = *(const CK_LDS u32x4*)(uintptr_t)(pa_k + i * 16 * RB);
+#pragma unroll
+                    for (int j = 0; j < JB; ++j) b[j] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + j * 16 * RB);
+#endif
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (burst_hi) __builtin_amdgcn_s_setprio(2);
+                    else __builtin_amdgcn_s_setprio(1);
+                    __builtin_amdgcn_sched_barrier(0);
+#if !defined(CK_PROBE_NO_SYNC)
                     if (ks == KSTEPS - 1 && JB == WTC) {
                         flag_add_after_reads(emptyA + fa_idx * 4);
                         flag_add(emptyB + fb_idx * 4);
                     }
+#endif
 #pragma unroll
                     for (int j = 0; j < WTC; ++j) {
+#if !defined(CK_PROBE_NO_SYNC)
                         if (ks == KSTEPS - 1 && JB != WTC && j == WTC - 1) {
                             flag_add_after_reads(emptyA + fa_idx * 4);
                             flag_add(emptyB + fb_idx * 4);
                         }
+#endif
 #pragma unroll
-                        for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(b[j % JB], a[i], acc[i][j]);
+                        for (int i = 0; i < WTR; ++i) {
+#if defined(CK_PROBE_NO_MFMA)  // measurement build only: consumers read fragments but skip the MFMAs
+                            asm volatile("" ::"v"(b[j % JB]), "v"(a[i]));
+#else
+                            acc[i][j] = MfmaOp<DT>::run(b[j % JB], a[i], acc[i][j]);
+#endif
+                        }
                         if (j + JB < WTC) {
+#if !defined(CK_PROBE_NO_SCHED_BARRIER)
                             __builtin_amdgcn_sched_barrier(0);
-                            b[j % JB] = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + (j + JB) * 16 * RB);
+#endif
+#if defined(CK_PROBE_NO_LDS)
+                            b[j % JB] = u32x4{pb_k, pb_k + j, 5u, 6u};
+#else
+                            b[j % JB] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + (j + JB) * 16 * RB);
+#endif
+#if !defined(CK_PROBE_NO_SCHED_BARRIER)
                             __builtin_amdgcn_sched_barrier(0);
+#endif
                         }
                     }
                 }
@@ -450,9 +541,8 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                             if (i == 0) wait_flag_ge(fb + j * 4, pb * (fill + 1), sp);
 #pragma unroll
                             for (int ks = 0; ks < KSTEPS; ++ks) {
-                                const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
-                                const u32x4 av = *(const CK_LDS u32x4*)(uintptr_t)(st + a_lane + coff + i * 16 * RB);
-                                const u32x4 bv = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + j * 16 * RB);
+                                const u32x4 av = *(const CK_LDS u32x4*)(uintptr_t)(((st + a_lane) ^ (uint32_t)(ks * 64)) + i * 16 * RB);
+                                const u32x4 bv = *(const CK_LDS u32x4*)(uintptr_t)(((st + b_lane) ^ (uint32_t)(ks * 64)) + j * 16 * RB);
                                 acc[i][j] = MfmaOp<DT>::run(bv, av, acc[i][j]);
                             }
                             if (i == WTR - 1) flag_add_after_reads(eb + j * 4);
@@ -468,16 +558,14 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                     u32x4 a[KSTEPS];
 #pragma unroll
                     for (int ks = 0; ks < KSTEPS; ++ks) {
-                        const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
-                        a[ks] = *(const CK_LDS u32x4*)(uintptr_t)(st + a_lane + coff + i * 16 * RB);
+                        a[ks] = *(const CK_LDS u32x4*)(uintptr_t)(((st + a_lane) ^ (uint32_t)(ks * 64)) + i * 16 * RB);
                     }
 #pragma unroll
                     for (int j = 0; j < WTC; ++j) {
                         if (j >= sb) {
 #pragma unroll
                             for (int ks = 0; ks < KSTEPS; ++ks) {
-                                const uint32_t coff = (uint32_t)(((ks * 4 + lg) ^ key) * CHUNK_BYTES);
-                                const u32x4 bv = *(const CK_LDS u32x4*)(uintptr_t)(st + b_lane + coff + j * 16 * RB);
+                                const u32x4 bv = *(const CK_LDS u32x4*)(uintptr_t)(((st + b_lane) ^ (uint32_t)(ks * 64)) + j * 16 * RB);
                                 acc[i][j] = MfmaOp<DT>::run(bv, a[ks], acc[i][j]);
                             }
                         }
@@ -492,10 +580,17 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
             if (++stage == S) { stage = 0; ++fill; }
         }
 
+#if defined(CK_PROBE_TIMING)
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
+            unsigned* o = g.status + 8 + (threadIdx.x >> 6) * 8;
+            o[0] = (unsigned)sp.wait_cycles; o[1] = (unsigned)(sp.wait_cycles >> 32); o[2] = sp.wait_calls; o[3] = sp.wait_polls;
+            o[4] = prefetch_hits;
+        }
+#endif
         // ---- epilogue: D = alpha * acc + beta * C straight from the accumulators. With the Bt
         // fragment as the first MFMA operand a lane holds 4 consecutive columns of one row.
-        const int m_base = rc.row * TILE + R * WTR * 16 + lr;
-        const int n_base = rc.col * TILE + Cc * WTC * 16 + lg * 4;
+        const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
+        const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
         const float alpha = g.alpha, beta = g.beta;
         const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
 #pragma unroll
@@ -531,17 +626,26 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_pc_kernel(const GemmArgs g) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
 
+    const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
     const int fregion = flag_region_bytes(MODE, CW, g.bar_steps_a, g.bar_steps_b, g.num_stages);
     for (int i = threadIdx.x; i < fregion / 4; i += blockDim.x) ((CK_LDS uint32_t*)ck_smem)[i] = 0;
     __syncthreads();
 
     const uint32_t flags_base = lds0, ring_base = lds0 + fregion;
+    // producers are rarely runnable and must issue their loads promptly when they are
+    if (wave < g.pa + g.pb) __builtin_amdgcn_s_setprio(3);
     if (wave < g.pa) {
         produce_px<TILE, SEGK, CW, MODE, true>(g, flags_base, ring_base, wave, g.pa, lane);
     } else if (wave < g.pa + g.pb) {
         produce_px<TILE, SEGK, CW, MODE, false>(g, flags_base, ring_base, wave - g.pa, g.pb, lane);
     } else if (wave < g.pa + g.pb + CW) {
         consume<DT, TILE, SEGK, CW, MODE>(g, flags_base, ring_base, wave - g.pa - g.pb, lane);
+        // the last consumer wave of workgroup 0 records how long the workgroup ran
+        if (blockIdx.x == 0 && threadIdx.x == blockDim.x - 1) {
+            const unsigned long long dc = clock64() - clk0, dw = wall_clock64() - wall0;
+            g.status[2] = (unsigned)dc; g.status[3] = (unsigned)(dc >> 32);
+            g.status[4] = (unsigned)dw; g.status[5] = (unsigned)(dw >> 32);
+        }
     }
 }
 

@@ -103,6 +103,17 @@ int ckopt_check_matmul_shmem_tuning(int tile_dim, int block_rows);
  * (cuda::barrier waits are unbounded). */
 int ckopt_device_status(void* stream);
 
+/* Waits for `stream`, then reports how long workgroup 0 of the last GEMM launch on the current device
+ * ran: shader-clock cycles and ticks of the constant 100 MHz reference clock. Their ratio is the clock
+ * the compute units actually ran at (it drops under matrix-core load), which turns a duration into a
+ * matrix-core utilisation. No reference counterpart. */
+int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* ref_ticks);
+
+/* Copies up to 128 words of per-wave cycle counters that measurement builds of the library
+ * (compiled with -DCK_PROBE_TIMING) record for workgroup 0: 8 words per wave - cycles spent in
+ * flag waits (lo, hi), wait calls, polls, read-ahead hits. All zero in the normal build. */
+int ckopt_probe_counters(void* stream, unsigned int* out, int nwords);
+
 /* Process-wide tuning switches that are not launcher parameters in the reference:
  * key 0: LDS XOR swizzle on/off (default 1); key 1: spin limit of bounded waits (default 1<<22);
  * key 2: number of XCDs assumed by the workgroup->tile remap (default 8; 1 disables the remap).
