@@ -15,6 +15,8 @@ namespace ck {
 CK_DECL_GEMM(launch_gemm_pc_f16_m0) CK_DECL_GEMM(launch_gemm_pc_f16_m1) CK_DECL_GEMM(launch_gemm_pc_f16_m2)
 CK_DECL_GEMM(launch_gemm_pc_bf16_m0) CK_DECL_GEMM(launch_gemm_pc_bf16_m1) CK_DECL_GEMM(launch_gemm_pc_bf16_m2)
 #undef CK_DECL_GEMM
+hipError_t launch_gemm_fused_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
+hipError_t launch_gemm_fused_bf16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_matmul_shmem(int dtype, int tile, int accs, bool bt, dim3 grid, hipStream_t s, const SimtArgs& a);
 }  // namespace ck
 
@@ -26,6 +28,8 @@ namespace {
 std::atomic<int> g_swizzle{1};
 std::atomic<int> g_spin_limit{1 << 22};
 std::atomic<int> g_num_xcd{8};
+std::atomic<int> g_prio_mode{0};
+std::atomic<int> g_producer_nap{0};
 
 constexpr int MAX_DEV = 64;
 std::mutex g_status_mutex;
@@ -78,6 +82,8 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float*
     a.num_xcd = g_num_xcd.load();
     a.vec_store = (N % 4 == 0) && !((uintptr_t)D & 15) && (beta == 0.f || !((uintptr_t)C & 15));
     a.spin_limit = (uint32_t)g_spin_limit.load();
+    a.prio_mode = g_prio_mode.load();
+    a.producer_nap = g_producer_nap.load();
     const int src = status_ptr_for_current_device(&a.status);
     if (src != CK_OK) return src;
 
@@ -88,7 +94,10 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float*
                                            t.bar_step_rows_b, t.num_stages, t.num_consumer_waves);
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
-    if (dtype == CK_DT_F16) {
+    if (t.num_producer_waves == 0) {
+        e = dtype == CK_DT_F16 ? launch_gemm_fused_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a)
+                               : launch_gemm_fused_bf16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a);
+    } else if (dtype == CK_DT_F16) {
         if (mode == 0) e = launch_gemm_pc_f16_m0(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
         if (mode == 1) e = launch_gemm_pc_f16_m1(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
         if (mode == 2) e = launch_gemm_pc_f16_m2(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
@@ -254,6 +263,8 @@ int ckopt_set_option(int key, int value) {
         case 0: return g_swizzle.exchange(value != 0);
         case 1: if (value < 1) return ck::CK_ERR_BAD_PARAM; return g_spin_limit.exchange(value);
         case 2: if (value < 1 || value > 64) return ck::CK_ERR_BAD_PARAM; return g_num_xcd.exchange(value);
+        case 3: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_prio_mode.exchange(value);
+        case 4: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_producer_nap.exchange(value);
         default: return ck::CK_ERR_BAD_PARAM;
     }
 }

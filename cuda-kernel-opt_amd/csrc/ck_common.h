@@ -165,7 +165,9 @@ CK_HD int check_gemm_tuning(const GemmTuning& t) {
     if (!(t.tile_dim == 64 || t.tile_dim == 128 || t.tile_dim == 256)) return CK_ERR_BAD_PARAM;
     if (!(t.segment_dim_k == 32 || t.segment_dim_k == 64 || t.segment_dim_k == 128)) return CK_ERR_BAD_PARAM;
     if (!(t.num_consumer_waves == 4 || t.num_consumer_waves == 8)) return CK_ERR_BAD_PARAM;
-    if (!(t.num_producer_waves == 2 || t.num_producer_waves == 4 || t.num_producer_waves == 8)) return CK_ERR_BAD_PARAM;
+    // 0 producer waves: every consumer wave also streams its share of the segments (fused variant)
+    if (!(t.num_producer_waves == 0 || t.num_producer_waves == 2 || t.num_producer_waves == 4 || t.num_producer_waves == 8))
+        return CK_ERR_BAD_PARAM;
     if (t.num_stages < 1 || t.num_stages > MAX_STAGES) return CK_ERR_BAD_PARAM;
     if (t.tile_group_m < 1 || t.num_cus < 1) return CK_ERR_BAD_PARAM;
     const int wtr = wave_tile_rows(t.tile_dim, t.num_consumer_waves), wtc = wave_tile_cols(t.tile_dim, t.num_consumer_waves);
@@ -178,6 +180,7 @@ CK_HD int check_gemm_tuning(const GemmTuning& t) {
         if (t.bar_steps_a < 0 || t.bar_steps_a >= wtr) return CK_ERR_BAD_PARAM;
         if (t.bar_steps_b < 0 || t.bar_steps_b >= wtc) return CK_ERR_BAD_PARAM;
     }
+    if (t.num_producer_waves == 0 && mode != CK_SYNC_TILE) return CK_ERR_NO_INSTANCE;  // fused variant: one signal pair per stage
     // 64 accumulator blocks (256 registers) leave no room for a second wave on the SIMD
     if (get_num_acc(t.tile_dim, t.num_consumer_waves) > 32) return CK_ERR_NO_INSTANCE;
     if (t.num_producer_waves + t.num_consumer_waves > max_waves_for(t.tile_dim, t.num_consumer_waves)) return CK_ERR_NO_INSTANCE;

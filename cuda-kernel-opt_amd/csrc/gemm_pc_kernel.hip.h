@@ -63,6 +63,8 @@ struct GemmArgs {
     int num_xcd;
     int vec_store;  // D (and C) 16-byte aligned with N % 4 == 0
     uint32_t spin_limit;
+    int prio_mode;      // 0: producers at raised priority; 1: also asymmetric consumer burst priorities per SIMD pair; 2: none
+    int producer_nap;   // s_sleep argument class of the producers' flag polling: 0 -> 1, 1 -> 4, 2 -> 16
     unsigned int* status;  // device words: [0] OR of CK_STATUS_* bits, [2..3] shader cycles and [4..5] 100 MHz
                            // ticks workgroup 0 spent in the last launch (actual-clock evidence)
 };
@@ -102,6 +104,19 @@ __device__ __forceinline__ void flag_add_after_reads(uint32_t lds_addr) {
 __device__ __forceinline__ void flag_add(uint32_t lds_addr) {
     uint32_t one = 1;
     asm volatile("s_mov_b64 exec, 1\n\tds_add_u32 %0, %1\n\ts_mov_b64 exec, -1" ::"v"(lds_addr), "v"(one) : "memory");
+}
+
+// Split counter read: issue now, collect later. A volatile load would be followed by an immediate
+// full wait; here the wave keeps issuing, and the collect is a counted wait the caller places where
+// the answer has had time to arrive. The collect carries the values as in/out operands so that no
+// use can be scheduled ahead of it.
+__device__ __forceinline__ uint32_t flag_read_issue(uint32_t lds_addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(lds_addr) : "memory");
+    return v;
+}
+__device__ __forceinline__ void flag_read_collect(uint32_t& a, uint32_t& b) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)::"memory");
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt_imm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -200,7 +215,7 @@ template <int DEPTH> struct SignalQueue {
 // "landed" signals oldest first (each needs only the loads up to that entry), so it never blocks
 // while holding back a signal the consumers need to make progress.
 template <int DEPTH>
-__device__ __forceinline__ void producer_wait(uint32_t addr, uint32_t target, SignalQueue<DEPTH>& q, Spin& sp) {
+__device__ __forceinline__ void producer_wait(uint32_t addr, uint32_t target, SignalQueue<DEPTH>& q, Spin& sp, int nap) {
     if (target == 0 || sp.dead) return;
     uint32_t n = 0;
 #if defined(CK_PROBE_TIMING)
@@ -217,7 +232,9 @@ __device__ __forceinline__ void producer_wait(uint32_t addr, uint32_t target, Si
             if ((threadIdx.x & 63) == 0) atomicOr(sp.status, sp.bit);
             break;
         }
-        __builtin_amdgcn_s_sleep(1);
+        if (nap == 0) __builtin_amdgcn_s_sleep(1);
+        else if (nap == 1) __builtin_amdgcn_s_sleep(4);
+        else __builtin_amdgcn_s_sleep(16);
     }
 }
 
@@ -305,23 +322,23 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
             for (int blk = 0; blk < NBLK; ++blk) {
                 // ---- wait until the consumers of the previous fill have released these rows
                 if (MODE == CK_SYNC_TILE) {
-                    producer_wait(fl + (empty_off + 0) * 4, CW * fill, sq, sp);
+                    producer_wait(fl + (empty_off + 0) * 4, CW * fill, sq, sp, g.producer_nap);
                 } else if (MODE == CK_SYNC_WAVE) {
                     const int s_own = IS_A ? sa : sb, s_oth = IS_A ? sb : sa;
                     const int oth_max = IS_A ? 2 : CW / 2;
                     const bool first_has_res = (s_own == 0 || s_oth < oth_max);
-                    if (blk == 0 && first_has_res && nres > 0) producer_wait(fl + (empty_off + s_own) * 4, nres * fill, sq, sp);
+                    if (blk == 0 && first_has_res && nres > 0) producer_wait(fl + (empty_off + s_own) * 4, nres * fill, sq, sp, g.producer_nap);
                     if (blk < s_own && s_oth > 0) {
-                        producer_wait(fl + (empty_off + blk) * 4, s_oth * fill, sq, sp);
+                        producer_wait(fl + (empty_off + blk) * 4, s_oth * fill, sq, sp, g.producer_nap);
                     } else if (blk == s_own && !first_has_res && nres > 0) {
-                        producer_wait(fl + (empty_off + s_own) * 4, nres * fill, sq, sp);
+                        producer_wait(fl + (empty_off + s_own) * 4, nres * fill, sq, sp, g.producer_nap);
                     }
                 } else {
                     constexpr int WT = IS_A ? WTR : WTC;
                     const int s_own = IS_A ? sa : sb;
                     const int unit = blk / WT, sub = blk % WT;
                     const int readers = IS_A ? 2 : CW / 2;
-                    if (sub <= s_own) producer_wait(fl + (empty_off + unit * (s_own + 1) + sub) * 4, readers * fill, sq, sp);
+                    if (sub <= s_own) producer_wait(fl + (empty_off + unit * (s_own + 1) + sub) * 4, readers * fill, sq, sp, g.producer_nap);
                 }
                 // ---- this wave's share of the row block, straight into LDS
 #if defined(CK_PROBE_NO_LOADS)  // measurement build only: producers signal without loading
@@ -443,6 +460,7 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                 // The two "full" counters of this segment were read one segment ahead (behind the
                 // previous segment's fragment reads); poll only if they were not there yet.
 #if !defined(CK_PROBE_NO_SYNC)
+                flag_read_collect(pre_a, pre_b);
                 const uint32_t seen_a = __builtin_amdgcn_readfirstlane(pre_a);
                 const uint32_t seen_b = __builtin_amdgcn_readfirstlane(pre_b);
                 if ((int32_t)(seen_a - pa * (fill + 1)) < 0) wait_flag_ge(fullA + fa_idx * 4, pa * (fill + 1), sp);
@@ -454,8 +472,8 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                 {
                     const int nstage = stage + 1 == S ? 0 : stage + 1;
                     const uint32_t nfl = flags_base + (uint32_t)nstage * fps * 4;
-                    pre_a = *(volatile CK_LDS uint32_t*)(uintptr_t)(nfl + fa_idx * 4);
-                    pre_b = *(volatile CK_LDS uint32_t*)(uintptr_t)(nfl + 2 * ua * 4 + fb_idx * 4);
+                    pre_a = flag_read_issue(nfl + fa_idx * 4);
+                    pre_b = flag_read_issue(nfl + 2 * ua * 4 + fb_idx * 4);
                 }
 #endif
 #pragma unroll
@@ -471,7 +489,7 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                     // of them wins the matrix core outright, finishes its burst first and loads its next
                     // fragments while the other bursts, so the pair settles into ping-pong instead of
                     // stalling on LDS latency in lockstep.
-                    __builtin_amdgcn_s_setprio(0);
+                    if (g.prio_mode == 1) __builtin_amdgcn_s_setprio(0);
 #if defined(CK_PROBE_NO_LDS)  // measurement build only: fragments are made up in registers
 #pragma unroll
                     for (int i = 0; i < WTR; ++i) a[i] = u32x4{pa_k, pa_k + i, 1u, 2u};
@@ -484,8 +502,10 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                     for (int j = 0; j < JB; ++j) b[j] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + j * 16 * RB);
 #endif
                     __builtin_amdgcn_sched_barrier(0);
-                    if (burst_hi) __builtin_amdgcn_s_setprio(2);
-                    else __builtin_amdgcn_s_setprio(1);
+                    if (g.prio_mode == 1) {
+                        if (burst_hi) __builtin_amdgcn_s_setprio(2);
+                        else __builtin_amdgcn_s_setprio(1);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
 #if !defined(CK_PROBE_NO_SYNC)
                     if (ks == KSTEPS - 1 && JB == WTC) {
@@ -633,7 +653,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_pc_kernel(const GemmArgs g) {
 
     const uint32_t flags_base = lds0, ring_base = lds0 + fregion;
     // producers are rarely runnable and must issue their loads promptly when they are
-    if (wave < g.pa + g.pb) __builtin_amdgcn_s_setprio(3);
+    if (wave < g.pa + g.pb && g.prio_mode != 2) __builtin_amdgcn_s_setprio(3);
     if (wave < g.pa) {
         produce_px<TILE, SEGK, CW, MODE, true>(g, flags_base, ring_base, wave, g.pa, lane);
     } else if (wave < g.pa + g.pb) {

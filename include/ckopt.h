@@ -41,7 +41,9 @@ enum {
  * synchronisation granularity exactly as in the reference: (tile_dim, tile_dim), or
  * (wave_tile_rows*16, wave_tile_cols*16) with bar_steps_a <= C/2 and bar_steps_b <= 2, or (16, 16)
  * with bar_steps_a < wave_tile_rows and bar_steps_b < wave_tile_cols; num_producer_waves in
- * {2,4,8} (half stream A, half stream Bt); num_consumer_waves in {4,8}; num_cus = persistent grid.
+ * {2,4,8} (half stream A, half stream Bt) or 0 (no dedicated producers: every consumer wave also
+ * streams its share of each segment; tile granularity only); num_consumer_waves in {4,8};
+ * num_cus = persistent grid.
  * M, N need not be multiples of tile_dim and K need not be a multiple of segment_dim_k (edges are
  * zero-filled / masked), but K must be a multiple of 8 so that rows are 16-byte aligned. */
 int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* Bt, const float* C, float* D,
