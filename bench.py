@@ -84,6 +84,9 @@ def main():
     ap.add_argument("--cus", type=int, default=0, help="persistent grid size (default: all compute units)")
     ap.add_argument("--block-rows", type=int, default=2, help="matmul_shmem: block_rows (SIMT workload only)")
     ap.add_argument("--simt-tile", type=int, default=128)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain 1 GiB device copy kernel (reads 1 GiB, writes 1 GiB): the reference "
+                         "reading for FETCH_SIZE / WRITE_SIZE counter runs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
@@ -102,6 +105,16 @@ def main():
     ck = load_package()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        n = 1 << 28  # fp32 elements: 1 GiB
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(max(args.steps, 1)):
+            torch.add(src, 1.0, out=dst)  # one elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "elementwise copy kernel", "bytes_read": n * 4, "bytes_written": n * 4,
+                          "launches": max(args.steps, 1)}))
+        return 0
     cus = args.cus or torch.cuda.get_device_properties(0).multi_processor_count
 
     kind, dtype, M, N, K, dist = WORKLOADS[args.workload]

@@ -211,6 +211,38 @@ def test_ragged_edges_aligned_k(ck, oracle, M, N, K):
             assert np.array_equal(got, (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32))
 
 
+@pytest.mark.parametrize("tile,c", [(64, 4), (64, 8), (128, 4), (128, 8), (256, 8)])
+def test_fused_variant_no_producer_waves(ck, oracle, tile, c):
+    # num_producer_waves == 0: every wave loads its share and multiplies; exact on small integers for every
+    # segment size and ring depth (1 and 2 stages exercise the late-signal / late-refill paths), ragged too
+    a = ck.fill_int(ck.DT_F16, (2 * tile, 640), 51, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (3 * tile, 640), 51, 1, -2, 2)
+    want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)
+    ar = ck.fill_int(ck.DT_F16, (tile + 40, 72), 51, 2, -2, 2)
+    br = ck.fill_int(ck.DT_F16, (tile - 24, 72), 51, 3, -2, 2)
+    wantr = (ar.astype(np.int64) @ br.astype(np.int64).T).astype(np.float32)
+    n = 0
+    for sk in (32, 64, 128):
+        for stages in (1, 2, 3, 4, 6):
+            t = make_tuning(ck, tile, sk, stages, 0, c)
+            if not legal(ck, t):
+                continue
+            assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want), t
+            assert np.array_equal(G.run_gemm(ck, ck.DT_F16, ar, br, t=t), wantr), t
+            n += 1
+    assert n >= 8
+    # granularities other than tile have no fused instance
+    t = make_tuning(ck, tile, 32, 2, 0, c, "wave", 1, 1)
+    assert not legal(ck, t)
+    # random data, alpha/beta, bf16
+    M, N, K = 2 * tile, 2 * tile, 1024
+    a2 = ck.fill_uniform(ck.DT_BF16, (M, K), 52, 0)
+    b2 = ck.fill_uniform(ck.DT_BF16, (N, K), 52, 1)
+    c2 = ck.fill_uniform(ck.DT_F32, (M, N), 52, 2)
+    ref = oracle.gemm(oracle.DT_BF16, a2, b2, c2, 1.5, -0.5)
+    assert_close(oracle, ref, G.run_gemm(ck, ck.DT_BF16, a2, b2, c2, 1.5, -0.5, t=make_tuning(ck, tile, 32, 4, 0, c)))
+
+
 def test_port_0_and_port_1_entry_points(ck):
     M, N, K = 256, 384, 512
     a = ck.fill_int(ck.DT_F16, (M, K), 41, 0, -2, 2)
