@@ -265,8 +265,8 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         // first MFMA must not see newer LDS operations, or it would wait for them as well
         acc[0][0] = MfmaOp<DT>::run(fb[P][0], fa[P][0], acc[0][0]);
         __builtin_amdgcn_sched_barrier(0);
-        uint32_t s_full = flag_read_issue(full_addr(n_stage));
-        uint32_t s_empty = flag_read_issue(empty_addr(l_stage));
+        uint32_t s_full = flag_peek(full_addr(n_stage));
+        uint32_t s_empty = flag_peek(empty_addr(l_stage));
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < WTC / 2; ++j)
@@ -275,7 +275,6 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
                 if (i + j > 0) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
             }
         __builtin_amdgcn_sched_barrier(0);
-        flag_read_collect(s_full, s_empty);
         if (refill_now) {
             if (l_fill > 0 && (int32_t)(__builtin_amdgcn_readfirstlane(s_empty) - (uint32_t)CW * l_fill) < 0)
                 wait_flag_ge(empty_addr(l_stage), (uint32_t)CW * l_fill, sp);

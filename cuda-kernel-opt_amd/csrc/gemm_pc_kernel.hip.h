@@ -106,17 +106,13 @@ __device__ __forceinline__ void flag_add(uint32_t lds_addr) {
     asm volatile("s_mov_b64 exec, 1\n\tds_add_u32 %0, %1\n\ts_mov_b64 exec, -1" ::"v"(lds_addr), "v"(one) : "memory");
 }
 
-// Split counter read: issue now, collect later. A volatile load would be followed by an immediate
-// full wait; here the wave keeps issuing, and the collect is a counted wait the caller places where
-// the answer has had time to arrive. The collect carries the values as in/out operands so that no
-// use can be scheduled ahead of it.
-__device__ __forceinline__ uint32_t flag_read_issue(uint32_t lds_addr) {
-    uint32_t v;
-    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(lds_addr) : "memory");
-    return v;
-}
-__device__ __forceinline__ void flag_read_collect(uint32_t& a, uint32_t& b) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b)::"memory");
+// Counter read whose answer is needed later: a relaxed workgroup-scope atomic load compiles to a
+// plain ds_read_b32 that the compiler's wait-count pass tracks, so the wave keeps issuing and the
+// (counted) wait lands at the first use of the value. The read must stay visible to the compiler:
+// an inline-asm read would leave it free to copy or spill the destination register before the
+// data has arrived.
+__device__ __forceinline__ uint32_t flag_peek(uint32_t lds_addr) {
+    return __hip_atomic_load((const CK_LDS uint32_t*)(uintptr_t)lds_addr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
 template <int N> __device__ __forceinline__ void wait_vmcnt_imm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -460,7 +456,6 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                 // The two "full" counters of this segment were read one segment ahead (behind the
                 // previous segment's fragment reads); poll only if they were not there yet.
 #if !defined(CK_PROBE_NO_SYNC)
-                flag_read_collect(pre_a, pre_b);
                 const uint32_t seen_a = __builtin_amdgcn_readfirstlane(pre_a);
                 const uint32_t seen_b = __builtin_amdgcn_readfirstlane(pre_b);
                 if ((int32_t)(seen_a - pa * (fill + 1)) < 0) wait_flag_ge(fullA + fa_idx * 4, pa * (fill + 1), sp);
@@ -472,8 +467,8 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                 {
                     const int nstage = stage + 1 == S ? 0 : stage + 1;
                     const uint32_t nfl = flags_base + (uint32_t)nstage * fps * 4;
-                    pre_a = flag_read_issue(nfl + fa_idx * 4);
-                    pre_b = flag_read_issue(nfl + 2 * ua * 4 + fb_idx * 4);
+                    pre_a = flag_peek(nfl + fa_idx * 4);
+                    pre_b = flag_peek(nfl + 2 * ua * 4 + fb_idx * 4);
                 }
 #endif
 #pragma unroll
