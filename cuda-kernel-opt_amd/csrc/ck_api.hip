@@ -90,8 +90,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float*
     const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
     const int grid = (int)(tiles < t.num_cus ? tiles : t.num_cus);
     const dim3 block((t.num_producer_waves + t.num_consumer_waves) * WAVE);
-    const size_t lds = (size_t)get_lds_req(t.tile_dim, t.segment_dim_k, a.bar_steps_a, a.bar_steps_b, t.bar_step_rows_a,
-                                           t.bar_step_rows_b, t.num_stages, t.num_consumer_waves);
+    const size_t lds = (size_t)gemm_lds_bytes(t);
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
     if (t.num_producer_waves == 0) {

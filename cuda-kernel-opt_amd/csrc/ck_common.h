@@ -161,6 +161,13 @@ struct GemmTuning {
 // per-wave register budget: all waves of a kernel get the same allocation out of 512 per SIMD lane.
 CK_HD int max_waves_for(int tile_dim, int /*consumer_waves*/) { return tile_dim == 256 ? 12 : 16; }
 
+// Dynamic LDS of a launch. The fused variant keeps no counters in LDS: the whole allocation is ring.
+CK_HD int gemm_lds_bytes(const GemmTuning& t) {
+    if (t.num_producer_waves == 0) return t.num_stages * 2 * stage_bytes_one_operand(t.tile_dim, t.segment_dim_k);
+    return get_lds_req(t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b, t.bar_step_rows_a, t.bar_step_rows_b,
+                       t.num_stages, t.num_consumer_waves);
+}
+
 CK_HD int check_gemm_tuning(const GemmTuning& t) {
     if (!(t.tile_dim == 64 || t.tile_dim == 128 || t.tile_dim == 256)) return CK_ERR_BAD_PARAM;
     if (!(t.segment_dim_k == 32 || t.segment_dim_k == 64 || t.segment_dim_k == 128)) return CK_ERR_BAD_PARAM;
@@ -180,12 +187,13 @@ CK_HD int check_gemm_tuning(const GemmTuning& t) {
         if (t.bar_steps_a < 0 || t.bar_steps_a >= wtr) return CK_ERR_BAD_PARAM;
         if (t.bar_steps_b < 0 || t.bar_steps_b >= wtc) return CK_ERR_BAD_PARAM;
     }
-    if (t.num_producer_waves == 0 && mode != CK_SYNC_TILE) return CK_ERR_NO_INSTANCE;  // fused variant: one signal pair per stage
+    // fused variant: the waves meet at the workgroup barrier once per segment (no finer granularity),
+    // and a stage is refilled while the next one is multiplied, so it needs at least two
+    if (t.num_producer_waves == 0 && (mode != CK_SYNC_TILE || t.num_stages < 2)) return CK_ERR_NO_INSTANCE;
     // 64 accumulator blocks (256 registers) leave no room for a second wave on the SIMD
     if (get_num_acc(t.tile_dim, t.num_consumer_waves) > 32) return CK_ERR_NO_INSTANCE;
     if (t.num_producer_waves + t.num_consumer_waves > max_waves_for(t.tile_dim, t.num_consumer_waves)) return CK_ERR_NO_INSTANCE;
-    const int lds = get_lds_req(t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b, t.bar_step_rows_a,
-                                t.bar_step_rows_b, t.num_stages, t.num_consumer_waves);
+    const int lds = gemm_lds_bytes(t);
     if (lds > LDS_BYTES_PER_CU) return CK_ERR_LDS_BUDGET;
     return CK_OK;
 }

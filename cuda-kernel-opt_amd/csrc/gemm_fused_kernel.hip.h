@@ -1,20 +1,31 @@
-// gemm_shmem_tc_async_opt_port with num_producer_waves == 0: the same LDS ring, direct-to-LDS loads,
-// MFMA wave tiles and flag counters as the producer/consumer kernel, but every wave is both: it
-// streams its 1/CW share of each K-segment into the ring and multiplies out of it.
+// gemm_shmem_tc_async_opt_port with num_producer_waves == 0: the same LDS ring, direct-to-LDS loads
+// and MFMA wave tiles as the producer/consumer kernel, but every wave is both. It streams its 1/CW
+// share of each K-segment into the ring and multiplies out of it, and the waves of a workgroup meet
+// at the hardware workgroup barrier once per segment instead of exchanging flag counters.
 //
 // Why this variant exists: all waves of a kernel get the same register allocation, so dedicated
 // producer waves push a 256 x 256 tile (8 consumer waves, 128 accumulator registers each) to three
 // waves per SIMD and 168 registers per wave - no room to hold the next k-step's fragments while the
-// current one is being multiplied, and the LDS latency of every k-step is exposed unless the
-// partner wave happens to cover it. With 8 waves (two per SIMD) each wave has 256 registers: the
-// fragments are double-buffered in registers, the loads of k-step t+1 are issued before the MFMAs of
-// k-step t, and flag waits fall behind a whole k-step of matrix-core work.
+// current one is being multiplied. With 8 waves (two per SIMD) each wave has 256 registers: the
+// fragments are double-buffered in registers and the LDS reads of k-step t+1 are issued under the
+// MFMAs of k-step t.
 //
-// Per stage two counters: full (+1 per wave once ITS loads into the stage have landed; vmcnt on the
-// wave's in-order queue) and empty (+1 per wave once the stage's fragments are in ITS registers).
-// Segment X is loaded S-1 segments before it is multiplied, its "landed" signal is sent one segment
-// before its fragments are first wanted, and when a stage is not full yet at prefetch time the wave
-// multiplies first and fetches afterwards instead of stalling in front of the matrix core.
+// Schedule of one wave (segment G, k-steps 0 .. KSTEPS-1, fragments of a k-step fetched one k-step
+// ahead):
+//   at the segment's LAST k-step, once its fragments are in registers:
+//     wait until this wave's own loads of segment G+1 have landed (in-order vmcnt),
+//     a few MFMAs that need registers only, then the workgroup barrier. Behind the barrier
+//       (a) every wave's share of segment G+1 is in LDS  -> its fragments may be fetched, and
+//       (b) every wave holds the last fragments of segment G -> its stage is free,
+//     so the wave issues its loads of segment G+S into that stage (S-1 segments of slack before
+//     they are wanted) and fetches the first fragments of segment G+1 under the remaining MFMAs.
+// The stream of segments runs across the tiles of the persistent workgroup: the loads of the next
+// tile are in flight while the current one is finished and written out.
+//
+// The direct-to-LDS loads are issued from inline assembly. The compiler cannot tell which LDS bytes
+// such a load will write, so with the builtin it drains ALL outstanding loads (vmcnt 0) in front of
+// every LDS read of the wave - which would serialise global latency into every k-step. Which loads
+// must have landed before which LDS read is exactly what the barrier protocol above establishes.
 #ifndef CK_GEMM_FUSED_KERNEL_HIP_H
 #define CK_GEMM_FUSED_KERNEL_HIP_H
 
@@ -22,9 +33,56 @@
 
 #include "gemm_pc_kernel.hip.h"
 
+// columns of 16 x 16 blocks multiplied between the landing wait and the barrier
+#ifndef CK_FUSED_PRE_COLS
+#define CK_FUSED_PRE_COLS 1
+#endif
+
 namespace ck {
 
-template <int N> __device__ __forceinline__ void wait_lgkmcnt_imm() { asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory"); }
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane from a raw buffer straight into LDS at lds_dst + lane * 16. voff is range
+// checked against the descriptor (out of range lanes write zeros), soff is not.
+__device__ __forceinline__ void dma_load_b128(i32x4 rsrc, uint32_t lds_dst, uint32_t voff, uint32_t soff) {
+#if defined(CK_PROBE_NO_LOADS)  // measurement build only: nothing is loaded
+    return;
+#endif
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory");
+}
+__device__ __forceinline__ i32x4 make_rsrc(const void* base, uint32_t num_records) {
+    const uint64_t p = (uint64_t)(uintptr_t)base;
+    i32x4 r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((p >> 32) & 0xffffu));  // stride 0: raw buffer
+    r[2] = __builtin_amdgcn_readfirstlane((int)num_records);
+    r[3] = 0x00020000;
+    return r;
+}
+// workgroup barrier that the compiler treats as a full memory clobber (no LDS access moves across)
+#if defined(CK_PROBE_NO_BARRIER)  // measurement build only (results are wrong without the barrier)
+__device__ __forceinline__ void wg_barrier() { asm volatile("" ::: "memory"); }
+#else
+__device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" ::: "memory"); }
+#endif
+__device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+template <int N> __device__ __forceinline__ void use_fragment_array(const u32x4 (&f)[N]) {
+    if constexpr (N == 8) asm volatile("" ::"v"(f[0]), "v"(f[1]), "v"(f[2]), "v"(f[3]), "v"(f[4]), "v"(f[5]), "v"(f[6]), "v"(f[7]) : "memory");
+    else if constexpr (N == 4) asm volatile("" ::"v"(f[0]), "v"(f[1]), "v"(f[2]), "v"(f[3]) : "memory");
+    else if constexpr (N == 2) asm volatile("" ::"v"(f[0]), "v"(f[1]) : "memory");
+    else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) asm volatile("" ::"v"(f[i]) : "memory");
+    }
+}
+template <int NA, int NB> __device__ __forceinline__ void use_fragments(const u32x4 (&a)[NA], const u32x4 (&b)[NB]) {
+    use_fragment_array(a);
+    use_fragment_array(b);
+}
 
 template <typename DT, int TILE, int SEGK, int CW>
 __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
@@ -37,118 +95,93 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
     constexpr int NI = TILE / RPI;             // wave loads per operand stage
     constexpr int LPW = 2 * NI / CW;           // wave loads per wave and stage
     constexpr bool STATIC_SPLIT = NI % CW == 0;  // the first LPW/2 loads of a wave are A, the rest Bt
+    constexpr int HALF = NI / CW > 0 ? NI / CW : 1;
     constexpr int VAR = CPR == 4 ? 1 : CPR == 8 ? 2 : 4;
-    static_assert(2 * NI % CW == 0 && LPW >= 1, "stage must split evenly over the waves");
+    constexpr int LPK = LPW / KSTEPS;          // wave loads per wave and k-step
+    constexpr int PRE = CK_FUSED_PRE_COLS < WTC ? CK_FUSED_PRE_COLS : WTC - 1;
+    static_assert(2 * NI % CW == 0 && LPW >= 1 && LPK * KSTEPS == LPW && LPK >= 1, "stage must split evenly over waves and k-steps");
 
     extern __shared__ __attribute__((aligned(1024))) char ck_smem[];
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(CK_LDS char*)ck_smem;
+    const uint32_t ring_base = (uint32_t)(uintptr_t)(CK_LDS char*)ck_smem;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
 
     const int S = g.num_stages;
-    const int fregion = flag_region_bytes(CK_SYNC_TILE, CW, 0, 0, S);
-    for (int i = threadIdx.x; i < fregion / 4; i += blockDim.x) ((CK_LDS uint32_t*)ck_smem)[i] = 0;
-    __syncthreads();
-    const uint32_t flags_base = lds0, ring_base = lds0 + fregion;
-    // per stage: [full, empty]
-    auto full_addr = [&](int stage) { return flags_base + (uint32_t)stage * 8u; };
-    auto empty_addr = [&](int stage) { return flags_base + (uint32_t)stage * 8u + 4u; };
-
     const int grid = gridDim.x;
     const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
     const int total_tiles = g.tiles_m * g.tiles_n;
     const int my_tiles = slot < total_tiles ? (total_tiles - slot + grid - 1) / grid : 0;
     const int nseg = g.nseg;
     const int total_segs = my_tiles * nseg;
-    Spin sp{g.spin_limit, g.status, CK_STATUS_CONSUMER_TIMEOUT, false};
 
-    // ---- loader side: which segment this wave issues next, descriptors of that segment's tile ------
+    // ---- loader side -----------------------------------------------------------------------------------
+    // A wave load E covers rows [E*RPI, (E+1)*RPI) of an operand stage; lane (lane_row, lane_slot)
+    // fetches the 16-byte chunk that belongs at its linear LDS slot under the XOR swizzle. Wave w
+    // issues the loads E = w, w + CW, ... of A and then of Bt (with fewer loads than waves: one load of
+    // one operand). CW is a multiple of the swizzle key's period in E, so one per-lane offset serves
+    // all loads of a wave. The loads of a segment are issued in KSTEPS chunks of LPK loads, one chunk
+    // per k-step and inside it one load every few MFMA columns: eight waves that issue all their
+    // loads back to back right behind the barrier queue up at the CU's one address unit and stall in
+    // front of their MFMAs.
     const uint32_t pitch32 = (uint32_t)g.K * 2u;
     const int lane_row = lane / CPR, lane_slot = lane % CPR;
-    uint32_t lane_off[VAR];
-    int lane_chunk[VAR];
-#pragma unroll
-    for (int v = 0; v < VAR; ++v) {
-        lane_chunk[v] = swizzle_slot(v * RPI + lane_row, lane_slot, CPR, g.swizzle);
-        lane_off[v] = (uint32_t)lane_row * pitch32 + (uint32_t)lane_chunk[v] * CHUNK_BYTES;
-    }
+    const int lchunk_w = swizzle_slot((wave % VAR) * RPI + lane_row, lane_slot, CPR, g.swizzle);
+    const uint32_t loff_w = (uint32_t)lane_row * pitch32 + (uint32_t)lchunk_w * CHUNK_BYTES;
     const uint32_t load_step = (uint32_t)RPI * pitch32;
     int l_tc = slot, l_seg = 0, l_stage = 0;
-    uint32_t l_fill = 0;
-    int issued_segs = 0;     // segments this wave has issued loads for
-    int signalled = 0;       // segments whose "landed" signal this wave has sent
-    __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b;
+    int opened_segs = 0;       // segments whose first chunk has been issued
+    int issued_loads = 0;      // loads this wave has issued so far
+    i32x4 rsrc_a = {0, 0, 0, 0}, rsrc_b = {0, 0, 0, 0};
     uint32_t nrec_a = 0, nrec_b = 0;
-    bool full_a = false, full_b = false;
+    // the segment being issued
+    uint32_t ld_base = 0, ld_k0x2 = 0;
+    bool ld_ktail = false;
 
-    auto open_tile = [&]() {
+    auto open_tile = [&]() __attribute__((always_inline)) {
+#if defined(CK_PROBE_SAME_TILE)  // measurement build only: every workgroup loads the operands of tile (0, 0)
+        const TileRC rc{0, 0};
+#elif defined(CK_PROBE_SAME_ROW)  // measurement build only: every workgroup loads A of tile row 0
+        const TileRC rc{0, tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, l_tc).col};
+#else
         const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, l_tc);
+#endif
         const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE);
         const int ra = g.M - row_a < TILE ? g.M - row_a : TILE, rb = g.N - row_b < TILE ? g.N - row_b : TILE;
         nrec_a = (uint32_t)ra * pitch32;
         nrec_b = (uint32_t)rb * pitch32;
-        full_a = ra == TILE;
-        full_b = rb == TILE;
-        rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)g.A + (int64_t)row_a * pitch32), 0, (int)nrec_a, 0x00020000);
-        rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)g.Bt + (int64_t)row_b * pitch32), 0, (int)nrec_b, 0x00020000);
+        rsrc_a = make_rsrc((const char*)g.A + (int64_t)row_a * pitch32, nrec_a);
+        rsrc_b = make_rsrc((const char*)g.Bt + (int64_t)row_b * pitch32, nrec_b);
     };
-
-    // issues this wave's LPW loads of segment `issued_segs` and advances the loader
-    auto issue_segment = [&]() {
+    // starts the next segment: its stage, its k offset, whether it reaches past K
+    auto open_segment = [&]() __attribute__((always_inline)) {
         if (l_seg == 0) open_tile();
-        const int k0 = l_seg * SEGK;
-        const uint32_t st_base = ring_base + (uint32_t)l_stage * (2 * OPB);
-        const bool k_full = k0 + SEGK <= g.K;
-#pragma unroll
-        for (int i = 0; i < LPW; ++i) {
-            const int e = wave + i * CW;  // index over the 2 * NI wave loads of the stage
-            const bool is_a = STATIC_SPLIT ? (i < NI / CW) : (e < NI);
-            const int E = STATIC_SPLIT ? (wave + (i % (NI / CW > 0 ? NI / CW : 1)) * CW) : (is_a ? e : e - NI);
-            const __amdgpu_buffer_rsrc_t rsrc = is_a ? rsrc_a : rsrc_b;
-            const uint32_t nrec = is_a ? nrec_a : nrec_b;
-            CK_LDS void* dst = (CK_LDS void*)(uintptr_t)(st_base + (is_a ? 0u : (uint32_t)OPB) + (uint32_t)E * 1024u);
-            uint32_t loff = lane_off[0];
-            int lchunk = lane_chunk[0];
-#pragma unroll
-            for (int v = 1; v < VAR; ++v) {
-                if (E % VAR == v) { loff = lane_off[v]; lchunk = lane_chunk[v]; }
-            }
-            if ((is_a ? full_a : full_b) && k_full) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, dst, 16, loff, (uint32_t)E * load_step + (uint32_t)k0 * 2u, 0, 0);
-            } else {
-                uint32_t voff = loff + (uint32_t)E * load_step + (uint32_t)k0 * 2u;
-                if (k0 + lchunk * CHUNK_ELEMS >= g.K) voff = nrec;  // absent k: zero fill
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, dst, 16, voff, 0, 0, 0);
-            }
-        }
-        ++issued_segs;
+        ld_base = ring_base + (uint32_t)l_stage * (2 * OPB);
+        ld_k0x2 = (uint32_t)l_seg * (SEGK * 2);
+        ld_ktail = (l_seg + 1) * SEGK > g.K;
+        ++opened_segs;
         if (++l_seg == nseg) { l_seg = 0; l_tc += grid; }
-        if (++l_stage == S) { l_stage = 0; ++l_fill; }
+        if (++l_stage == S) l_stage = 0;
     };
-    // my loads of segment `signalled` have landed when at most the later-issued ones are outstanding
-    int sig_stage = 0;       // stage of segment `signalled`
-#if defined(CK_PROBE_TIMING)
-    unsigned long long t_vm = 0, t_lgkm = 0, t_mid = 0;
-#define CK_T0() const unsigned long long ck_t0 = clock64()
-#define CK_T1(acc) acc += clock64() - ck_t0
-#else
-#define CK_T0()
-#define CK_T1(acc)
-#endif
-    auto signal_one = [&]() {
-        CK_T0();
-        const uint32_t later = (uint32_t)((issued_segs - 1 - signalled) * LPW);
-        if (later == LPW) wait_vmcnt_imm<LPW>();  // steady state with four stages
-        else if (later == 0) wait_vmcnt_imm<0>();
-        else wait_vmcnt_le(later);
-        CK_T1(t_vm);
-        flag_add(full_addr(sig_stage));
-        ++signalled;
-        if (++sig_stage == S) sig_stage = 0;
+    // load i (0 .. LPW-1) of the open segment. The whole global offset goes through the range-checked
+    // vector offset: rows past the tile edge and k past K land outside the descriptor and read as zero.
+    auto issue_load = [&](int i) __attribute__((always_inline)) {
+        bool is_a;
+        int E;
+        if (STATIC_SPLIT) {
+            is_a = i < HALF;
+            E = wave + (i % HALF) * CW;
+        } else {
+            is_a = wave < NI;
+            E = is_a ? wave : wave - NI;
+        }
+        uint32_t voff = loff_w + ((uint32_t)E * load_step + ld_k0x2);
+        if (ld_ktail && (int)(ld_k0x2 >> 1) + lchunk_w * CHUNK_ELEMS >= g.K) voff = is_a ? nrec_a : nrec_b;
+        dma_load_b128(is_a ? rsrc_a : rsrc_b, ld_base + (is_a ? 0u : (uint32_t)OPB) + (uint32_t)E * 1024u, voff, 0u);
+        ++issued_loads;
     };
 
-    // ---- consumer side -------------------------------------------------------------------------------
+    // ---- multiplier side -------------------------------------------------------------------------------
     const int R = wave / 2, Cc = wave % 2;
     const int lr = lane & 15, lg = lane >> 4;
     const int key = g.swizzle ? swizzle_key(lr, CPR) : 0;
@@ -162,147 +195,12 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < WTC; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto load_frags = [&](auto parity, int stage, int ks) {
-        constexpr int P = decltype(parity)::value;
-        const uint32_t st = ring_base + (uint32_t)stage * (2 * OPB);
-        const uint32_t pa_k = (st + a_lane) ^ (uint32_t)(ks * 64), pb_k = (st + b_lane) ^ (uint32_t)(ks * 64);
-#pragma unroll
-        for (int i = 0; i < WTR; ++i) fa[P][i] = *(const CK_LDS u32x4*)(uintptr_t)(pa_k + i * 16 * RB);
-#pragma unroll
-        for (int j = 0; j < WTC; ++j) fb[P][j] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + j * 16 * RB);
-    };
-
-    // prologue: fill S-1 stages (at least one), then fetch the fragments of k-step 0
-    for (int p = 0; p < (S > 1 ? S - 1 : 1) && issued_segs < total_segs; ++p) issue_segment();
-    if (total_segs > 0) {
-        signal_one();
-        wait_flag_ge(full_addr(0), (uint32_t)CW, sp);
-        asm volatile("" ::: "memory");
-        load_frags(std::integral_constant<int, 0>{}, 0, 0);
-    }
-
     int c_stage = 0;  // stage of the segment being multiplied
-    uint32_t c_fill = 0;
     int G = 0;        // index of the segment being multiplied, over all tiles of this workgroup
-
-    // ---- steady-state fast path ---------------------------------------------------------------------
-    // A wave issues roughly one instruction every four to five cycles, so next to the 32 MFMAs of a
-    // k-step (512 cycles) there is room for well under a hundred other instructions. kstep() above
-    // handles every case (stream start and end, tile changes of the loader, K tails, edge tiles, one
-    // or two stages) and is far heavier than that; kstep_fast() is the same protocol for a segment
-    // where nothing special happens: a next segment exists, the loader stays inside a full tile with
-    // all k present, it is exactly S-1 segments ahead and the signal for segment G+1 is due now.
-    // fast_run counts how many upcoming segments are known to be of that kind.
-    int fast_run = 0;
-    const uint32_t loff_w = lane_off[wave % VAR];  // CW is a multiple of VAR: a wave's loads share one key variant
-    const uint32_t wave_goff = (uint32_t)wave * load_step, cw_goff = (uint32_t)CW * load_step;
-    auto recompute_fast_run = [&]() {
-        fast_run = 0;
-        if (!STATIC_SPLIT || S < 3) return;
-        if (issued_segs != G + S - 1 || signalled != G + 1 || l_seg == 0 || !(full_a && full_b)) return;
-        int run = nseg - l_seg - ((g.K % SEGK) ? 1 : 0);
-        run = run < total_segs - issued_segs ? run : total_segs - issued_segs;
-        run = run < total_segs - 1 - G ? run : total_segs - 1 - G;
-        fast_run = run > 0 ? run : 0;
-    };
-    auto issue_fast = [&]() {
-        const uint32_t st_base = ring_base + (uint32_t)l_stage * (2 * OPB) + (uint32_t)wave * 1024u;
-        const uint32_t soff = (uint32_t)l_seg * (SEGK * 2) + wave_goff;
-        constexpr int HALF = NI / CW > 0 ? NI / CW : 1;
-#pragma unroll
-        for (int i = 0; i < LPW; ++i) {
-            const bool is_a = i < HALF;
-            const int ii = i % HALF;
-            CK_LDS void* dst = (CK_LDS void*)(uintptr_t)(st_base + (is_a ? 0u : (uint32_t)OPB) + (uint32_t)(ii * CW) * 1024u);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(is_a ? rsrc_a : rsrc_b, dst, 16, loff_w, soff + (uint32_t)ii * cw_goff, 0, 0);
-        }
-        ++issued_segs;
-        if (++l_seg == nseg) { l_seg = 0; l_tc += grid; }
-        if (++l_stage == S) { l_stage = 0; ++l_fill; }
-    };
-    // One k-step. Its fragments are in f[P] (possibly still arriving); the next k-step's go to f[1-P].
-    //   start : the fragments have arrived -> the stage is released if this is its last k-step; at a
-    //           segment's first k-step the "landed" signal of the next segment is sent
-    //   half 1: first MFMA, then the two counters this k-step depends on are sampled (the answers
-    //           arrive under the remaining MFMAs of the half)
-    //   middle: at a segment's first k-step the stage released one segment ago is refilled (after
-    //           making sure every wave has released it); the next fragments are fetched (after making
-    //           sure their stage is full); both waits are normally satisfied by the samples
-    //   half 2: second half of the MFMAs, covering the latency of what the middle issued
-    // `fast` selects the lean control path of a steady-state segment; the MFMA code is shared, so the
-    // accumulators stay in place whatever path the control sections take.
-    auto kstep = [&](auto parity, auto kstep_index, const bool fast) {
-        constexpr int P = decltype(parity)::value;
-        constexpr int KS = decltype(kstep_index)::value;
-        constexpr bool last_ks = KS == KSTEPS - 1;
-        int n_stage = c_stage;
-        uint32_t n_fill = c_fill;
-        if (last_ks) {
-            if (++n_stage == S) { n_stage = 0; ++n_fill; }
-        }
-        bool more = true, refill_now = KS == 0, need_full = last_ks;
-        wait_lgkmcnt_imm<0>();
-        if (last_ks) flag_add(empty_addr(c_stage));
-        if (fast) {
-            if (KS == 0) {
-                if (S == 4) wait_vmcnt_imm<LPW>();
-                else if (S == 3) wait_vmcnt_imm<0>();
-                else wait_vmcnt_le((uint32_t)((S - 3) * LPW));
-                flag_add(full_addr(sig_stage));
-                ++signalled;
-                if (++sig_stage == S) sig_stage = 0;
-            }
-        } else {
-            more = !(last_ks && G + 1 >= total_segs);  // is there a next k-step at all
-            // with two or more stages the ring is refilled at a segment's first k-step (the stage of the
-            // previous segment is free by then); with one the refill has to follow this segment's release
-            refill_now = (S >= 2 ? KS == 0 : last_ks) && issued_segs < total_segs && issued_segs - S <= (last_ks ? G : G - 1);
-            need_full = more && last_ks;
-            if (S >= 3 && KS == 0 && signalled <= G + 1 && signalled < issued_segs) signal_one();
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // first MFMA, then the two counter reads: the compiler's own fragment wait in front of the
-        // first MFMA must not see newer LDS operations, or it would wait for them as well
-        acc[0][0] = MfmaOp<DT>::run(fb[P][0], fa[P][0], acc[0][0]);
-        __builtin_amdgcn_sched_barrier(0);
-        uint32_t s_full = flag_peek(full_addr(n_stage));
-        uint32_t s_empty = flag_peek(empty_addr(l_stage));
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = 0; j < WTC / 2; ++j)
-#pragma unroll
-            for (int i = 0; i < WTR; ++i) {
-                if (i + j > 0) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
-            }
-        __builtin_amdgcn_sched_barrier(0);
-        if (refill_now) {
-            if (l_fill > 0 && (int32_t)(__builtin_amdgcn_readfirstlane(s_empty) - (uint32_t)CW * l_fill) < 0)
-                wait_flag_ge(empty_addr(l_stage), (uint32_t)CW * l_fill, sp);
-            if (fast) issue_fast();
-            else issue_segment();
-        }
-        if (more) {
-            if (need_full) {
-                if (!fast && S < 3) {
-                    // with one or two stages the next segment's signal cannot be sent any earlier
-                    while (signalled <= G + 1 && signalled < issued_segs) signal_one();
-                }
-                if ((int32_t)(__builtin_amdgcn_readfirstlane(s_full) - (uint32_t)CW * (n_fill + 1)) < 0)
-                    wait_flag_ge(full_addr(n_stage), (uint32_t)CW * (n_fill + 1), sp);
-            }
-            asm volatile("" ::: "memory");
-            load_frags(std::integral_constant<int, 1 - P>{}, last_ks ? n_stage : c_stage, last_ks ? 0 : KS + 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = WTC / 2; j < WTC; ++j)
-#pragma unroll
-            for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
-        __builtin_amdgcn_sched_barrier(0);
-    };
+    int seg_in_tile = 0, c_tc = slot;
 
     // ---- epilogue: D = alpha * acc + beta * C straight from the accumulators, then clear them
-    auto epilogue = [&](int tc) {
+    auto epilogue = [&](int tc) __attribute__((always_inline)) {
         const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
         const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
         const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
@@ -333,53 +231,190 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
             }
         }
     };
-    int seg_in_tile = 0, c_tc = slot;
-    auto end_segment = [&]() {
+
+    // this wave's loads of segment X have landed when at most the loads it issued after them are
+    // outstanding (a wave's loads complete in issue order; other memory operations in flight only
+    // make the wait longer, never shorter)
+    auto wait_landed = [&](int X) __attribute__((always_inline)) {
+        const int later = issued_loads - (X + 1) * LPW;
+        if (later == 2 * LPW) wait_vmcnt_imm<2 * LPW>();   // four stages in steady state
+        else if (later == LPW) wait_vmcnt_imm<LPW>();      // three stages
+        else if (later == 3 * LPW && 3 * LPW < 64) wait_vmcnt_imm<(3 * LPW < 64 ? 3 * LPW : 0)>();  // five stages
+        else if (later <= 0) wait_vmcnt_imm<0>();
+        else wait_vmcnt_le((uint32_t)later);
+    };
+
+#if defined(CK_PROBE_NO_MFMA)  // measurement build only: loads, waits and barriers without the multiplication
+#define CK_MFMA(b, a, c) (c)
+#else
+#define CK_MFMA(b, a, c) MfmaOp<DT>::run(b, a, c)
+#endif
+#if defined(CK_PROBE_TIMING)  // measurement build only: cycles in front of the LDS wait, the landing wait, the barrier
+    unsigned long long t_lds = 0, t_vm = 0, t_bar = 0;
+#define CK_T0() unsigned long long ck_t0 = clock64()
+#define CK_T1(acc) { const unsigned long long ck_t1 = clock64(); acc += ck_t1 - ck_t0; ck_t0 = ck_t1; }
+#else
+#define CK_T0()
+#define CK_T1(acc)
+#endif
+    // One k-step. Its fragments are in f[P] (possibly still arriving); the next k-step's go to f[1-P].
+    auto kstep = [&](auto parity, auto kstep_index) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity)::value;
+        constexpr int KS = decltype(kstep_index)::value;
+        constexpr bool last_ks = KS == KSTEPS - 1;
+        const bool has_next_seg = G + 1 < total_segs;
+        int n_stage = c_stage;
+        if (last_ks && ++n_stage == S) n_stage = 0;
+        const uint32_t st = ring_base + (uint32_t)(last_ks ? n_stage : c_stage) * (2 * OPB);
+        const uint32_t pa_k = (st + a_lane) ^ (uint32_t)((last_ks ? 0 : KS + 1) * 64);
+        const uint32_t pb_k = (st + b_lane) ^ (uint32_t)((last_ks ? 0 : KS + 1) * 64);
+
+        if (last_ks) {
+            CK_T0();
+            // The last fragments of this segment must be in registers before the barrier releases
+            // their stage. The wait is requested through a use of the registers the compiler can
+            // see: behind a bare s_waitcnt in inline assembly it would still count these reads as
+            // outstanding and pad every later fragment wait with the reads issued after the barrier.
+            use_fragments(fa[P], fb[P]);
+            CK_T1(t_lds);
+            if (has_next_seg) wait_landed(G + 1);
+            CK_T1(t_vm);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < PRE; ++j)
+#pragma unroll
+            for (int i = 0; i < WTR; ++i) acc[i][j] = CK_MFMA(fb[P][j], fa[P][i], acc[i][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        // chunk of LPK loads this k-step issues: at a segment's last k-step (behind the barrier) chunk 0
+        // of the segment that goes into the stage just released, otherwise the next chunk of the
+        // segment opened at the previous segment's last k-step
+        bool loading;
+        if (last_ks) {
+            loading = false;
+            if (has_next_seg) {
+                CK_T0();
+                wg_barrier();
+                CK_T1(t_bar);
+                if (opened_segs < total_segs) {
+                    open_segment();
+                    loading = true;
+                }
+            }
+        } else {
+            loading = issued_loads < opened_segs * LPW;
+        }
+        constexpr int CHUNK = last_ks ? 0 : KS + 1;
+        __builtin_amdgcn_sched_barrier(0);
+        // remaining columns; between them the fetch of the next k-step's fragments (A fragments
+        // first, then Bt) and this k-step's loads, one every LSTRIDE columns
+        constexpr int NF = WTR + WTC;                 // fragments to fetch
+        constexpr int COLS = WTC - PRE;               // columns left to multiply
+#if defined(CK_FUSED_FETCH_PER)
+        constexpr int PER = CK_FUSED_FETCH_PER;       // fetches per column (tuning builds)
+#else
+        constexpr int PER = (NF + COLS - 1) / COLS;   // fetches per column
+#endif
+        constexpr int LSTRIDE = COLS / LPK > 0 ? COLS / LPK : 1;
+#pragma unroll
+        for (int j = PRE; j < WTC; ++j) {
+            // (after the very last k-step of the stream this fetches fragments nobody uses: the
+            // addresses are inside the ring, and skipping them would put a branch in every column)
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                const int f = (j - PRE) * PER + q;
+#if !defined(CK_PROBE_NO_MFMA)
+                if (f < WTR) fa[1 - P][f] = *(const CK_LDS u32x4*)(uintptr_t)(pa_k + f * 16 * RB);
+                else if (f < NF) fb[1 - P][f - WTR] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + (f - WTR) * 16 * RB);
+#endif
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (loading) {
+#pragma unroll
+                for (int l = 0; l < LPK; ++l) {
+                    const int col = l * LSTRIDE < COLS ? l * LSTRIDE : COLS - 1;
+                    if (col == j - PRE) issue_load(CHUNK * LPK + l);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < WTR; ++i) acc[i][j] = CK_MFMA(fb[P][j], fa[P][i], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    bool tile_done = false;  // the segment just finished was the last of its tile: write it out
+    auto end_segment = [&]() __attribute__((always_inline)) {
         ++G;
-        if (++c_stage == S) { c_stage = 0; ++c_fill; }
+        if (++c_stage == S) c_stage = 0;
         if (++seg_in_tile == nseg) {
-            epilogue(c_tc);
             seg_in_tile = 0;
-            c_tc += grid;
+            tile_done = true;
         }
     };
 
-    // The two fragment buffers alternate per k-step. The stream of k-steps is walked in blocks of
-    // lcm(2, KSTEPS) k-steps so that buffer index and k-step index are compile-time constants inside
-    // a block: two segments per block when a segment is one k-step, one segment otherwise.
-    constexpr int SPB = KSTEPS == 1 ? 2 : 1;   // segments per block
-    using P0 = std::integral_constant<int, 0>;
-    using P1 = std::integral_constant<int, 1>;
-    while (G + SPB <= total_segs) {
-        const bool tile_end_inside = SPB == 2 && seg_in_tile + 1 == nseg;
-        const bool fast = fast_run >= SPB && !tile_end_inside;
-        if (fast) fast_run -= SPB;
-        if constexpr (KSTEPS == 1) {
-            kstep(P0{}, std::integral_constant<int, 0>{}, fast);
-            end_segment();
-            kstep(P1{}, std::integral_constant<int, 0>{}, fast);
-            end_segment();
-        } else {
-            kstep(P0{}, std::integral_constant<int, 0>{}, fast);
-            kstep(P1{}, std::integral_constant<int, 1>{}, fast);
-            if constexpr (KSTEPS == 4) {
-                kstep(P0{}, std::integral_constant<int, 2>{}, fast);
-                kstep(P1{}, std::integral_constant<int, 3>{}, fast);
-            }
-            end_segment();
+    if (total_segs > 0) {
+        // prologue: fill every stage, then fetch the fragments of k-step 0 once segment 0 is in LDS
+        for (int p = 0; p < S && opened_segs < total_segs; ++p) {
+            open_segment();
+#pragma unroll
+            for (int i = 0; i < LPW; ++i) issue_load(i);
         }
-        if (!fast) recompute_fast_run();
-    }
-    if (SPB == 2 && G < total_segs) {  // odd number of one-k-step segments: the last one
-        kstep(P0{}, std::integral_constant<int, 0>{}, false);
-        end_segment();
+        wait_landed(0);
+        wg_barrier();
+        {
+            const uint32_t pa_k = ring_base + a_lane, pb_k = ring_base + b_lane;
+#pragma unroll
+            for (int i = 0; i < WTR; ++i) fa[0][i] = *(const CK_LDS u32x4*)(uintptr_t)(pa_k + i * 16 * RB);
+#pragma unroll
+            for (int j = 0; j < WTC; ++j) fb[0][j] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + j * 16 * RB);
+        }
+
+        // The two fragment buffers alternate per k-step, and the buffer index is a compile-time
+        // constant: the loop body is one segment when that is an even number of k-steps, otherwise
+        // (one k-step per segment) two segments. A tile that ends between the two moves the fragments
+        // that were just fetched into buffer 0 and starts the body again, so there is one copy of
+        // the epilogue in the code.
+        using P0 = std::integral_constant<int, 0>;
+        using P1 = std::integral_constant<int, 1>;
+        using K0 = std::integral_constant<int, 0>;
+        using K1 = std::integral_constant<int, 1>;
+        using K2 = std::integral_constant<int, 2>;
+        using K3 = std::integral_constant<int, 3>;
+        for (;;) {
+            if (tile_done) {
+                epilogue(c_tc);
+                c_tc += grid;
+                tile_done = false;
+            }
+            if (G >= total_segs) break;
+            kstep(P0{}, K0{});
+            if constexpr (KSTEPS == 1) {
+                end_segment();
+                if (tile_done || G >= total_segs) {
+#pragma unroll
+                    for (int i = 0; i < WTR; ++i) fa[0][i] = fa[1][i];
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j) fb[0][j] = fb[1][j];
+                    continue;
+                }
+                kstep(P1{}, K0{});
+                end_segment();
+            } else {
+                kstep(P1{}, K1{});
+                if constexpr (KSTEPS == 4) {
+                    kstep(P0{}, K2{});
+                    kstep(P1{}, K3{});
+                }
+                end_segment();
+            }
+        }
     }
 
 #if defined(CK_PROBE_TIMING)
     if (blockIdx.x == 0 && lane == 0) {
         unsigned* o = g.status + 8 + wave * 8;
-        o[0] = (unsigned)sp.wait_cycles; o[1] = (unsigned)(sp.wait_cycles >> 32); o[2] = sp.wait_calls; o[3] = sp.wait_polls;
-        o[4] = (unsigned)(t_vm >> 4); o[5] = (unsigned)(t_lgkm >> 4); o[6] = (unsigned)(t_mid >> 4);
+        o[0] = (unsigned)t_vm; o[1] = (unsigned)(t_vm >> 32); o[2] = 0; o[3] = 0;
+        o[4] = (unsigned)(t_lds >> 4); o[5] = (unsigned)(t_vm >> 4); o[6] = (unsigned)(t_bar >> 4);
     }
 #endif
     if (blockIdx.x == 0 && threadIdx.x == blockDim.x - 1) {

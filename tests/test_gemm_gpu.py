@@ -214,7 +214,7 @@ def test_ragged_edges_aligned_k(ck, oracle, M, N, K):
 @pytest.mark.parametrize("tile,c", [(64, 4), (64, 8), (128, 4), (128, 8), (256, 8)])
 def test_fused_variant_no_producer_waves(ck, oracle, tile, c):
     # num_producer_waves == 0: every wave loads its share and multiplies; exact on small integers for every
-    # segment size and ring depth (1 and 2 stages exercise the late-signal / late-refill paths), ragged too
+    # segment size and ring depth, ragged too
     a = ck.fill_int(ck.DT_F16, (2 * tile, 640), 51, 0, -2, 2)
     bt = ck.fill_int(ck.DT_F16, (3 * tile, 640), 51, 1, -2, 2)
     want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)
@@ -223,14 +223,14 @@ def test_fused_variant_no_producer_waves(ck, oracle, tile, c):
     wantr = (ar.astype(np.int64) @ br.astype(np.int64).T).astype(np.float32)
     n = 0
     for sk in (32, 64, 128):
-        for stages in (1, 2, 3, 4, 6):
+        for stages in (1, 2, 3, 4, 5, 6):
             t = make_tuning(ck, tile, sk, stages, 0, c)
             if not legal(ck, t):
                 continue
             assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want), t
             assert np.array_equal(G.run_gemm(ck, ck.DT_F16, ar, br, t=t), wantr), t
             n += 1
-    assert n >= 6
+    assert n >= 5
     # granularities other than tile have no fused instance
     t = make_tuning(ck, tile, 32, 2, 0, c, "wave", 1, 1)
     assert not legal(ck, t)
