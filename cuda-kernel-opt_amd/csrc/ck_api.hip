@@ -49,6 +49,50 @@ int status_ptr_for_current_device(unsigned int** out) {
     return ck::CK_OK;
 }
 
+// Copies `rows` rows of K 2-byte elements into rows of Kp >= K elements (Kp % 8 == 0), zero filling
+// the tail: the form the direct-to-LDS loads need (every row starts on a 16-byte boundary). One
+// thread produces one 16-byte chunk of the destination from eight 2-byte reads.
+__global__ void pad_rows_kernel(const unsigned short* __restrict__ src, unsigned short* __restrict__ dst, int rows, int K, int Kp) {
+    const int chunks_per_row = Kp / 8;
+    const long long total = (long long)rows * chunks_per_row;
+    for (long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x; c < total; c += (long long)gridDim.x * blockDim.x) {
+        const int r = (int)(c / chunks_per_row), k0 = (int)(c % chunks_per_row) * 8;
+        const unsigned short* s = src + (long long)r * K + k0;
+        unsigned short v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = k0 + e < K ? s[e] : (unsigned short)0;
+        uint4 o;
+        o.x = v[0] | ((unsigned)v[1] << 16); o.y = v[2] | ((unsigned)v[3] << 16);
+        o.z = v[4] | ((unsigned)v[5] << 16); o.w = v[6] | ((unsigned)v[7] << 16);
+        *reinterpret_cast<uint4*>(dst + (long long)r * Kp + k0) = o;
+    }
+}
+
+int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta, int M,
+                int N, int K, const ck::GemmTuning& t, void* stream);
+
+// K % 8 != 0 or operands off a 16-byte boundary: the product is computed from zero-padded,
+// aligned copies of A and Bt in a stream-ordered temporary (zeros in the K tail add nothing).
+int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta,
+                         int M, int N, int K, const ck::GemmTuning& t, void* stream) {
+    using namespace ck;
+    const int Kp = (K + CHUNK_ELEMS - 1) / CHUNK_ELEMS * CHUNK_ELEMS;
+    const size_t bytes_a = (size_t)M * Kp * 2, bytes_b = (size_t)N * Kp * 2;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    void* ws = nullptr;
+    if (hipMallocAsync(&ws, bytes_a + bytes_b, s) != hipSuccess || !ws) return CK_ERR_HIP;
+    unsigned short* pa = static_cast<unsigned short*>(ws);
+    unsigned short* pb = pa + (size_t)M * Kp;
+    const int threads = 256;
+    auto blocks = [&](long long chunks) { long long b = (chunks + threads - 1) / threads; return (unsigned)(b < 65535 * 8 ? (b > 0 ? b : 1) : 65535 * 8); };
+    hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks((long long)M * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(A), pa, M, K, Kp);
+    hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks((long long)N * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(Bt), pb, N, K, Kp);
+    int rc = hipGetLastError() == hipSuccess ? CK_OK : CK_ERR_HIP;
+    if (rc == CK_OK) rc = gemm_launch(dtype, pa, pb, C, D, alpha, beta, M, N, Kp, t, stream);
+    if (hipFreeAsync(ws, s) != hipSuccess && rc == CK_OK) rc = CK_ERR_HIP;
+    return rc;
+}
+
 int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta, int M,
                 int N, int K, const ck::GemmTuning& t, void* stream) {
     using namespace ck;
@@ -58,9 +102,11 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float*
     if (rc != CK_OK) return rc;
     if (!A || !Bt || !D) return CK_ERR_NULL;
     if (beta != 0.f && !C) return CK_ERR_NULL;
-    if (K % CHUNK_ELEMS != 0) return CK_ERR_ALIGNMENT;  // rows must start on 16-byte boundaries
-    if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) return CK_ERR_ALIGNMENT;
+    if (((uintptr_t)A & 1) || ((uintptr_t)Bt & 1)) return CK_ERR_ALIGNMENT;
     if (((uintptr_t)D & 3) || ((uintptr_t)C & 3)) return CK_ERR_ALIGNMENT;
+    // the kernels want every operand row on a 16-byte boundary
+    if (K % CHUNK_ELEMS != 0 || ((uintptr_t)A & 15) || ((uintptr_t)Bt & 15))
+        return gemm_launch_repacked(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream);
     // one tile's rows are addressed through a 32-bit buffer offset
     if ((int64_t)t.tile_dim * K * 2 >= (int64_t)1 << 31) return CK_ERR_TOO_LARGE;
 

@@ -38,6 +38,11 @@
 #define CK_FUSED_PRE_COLS 1
 #endif
 
+// cache policy bits of the direct-to-LDS loads (tuning builds may set "nt", "sc0", "sc1")
+#ifndef CK_DMA_CPOL
+#define CK_DMA_CPOL ""
+#endif
+
 namespace ck {
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -48,7 +53,7 @@ __device__ __forceinline__ void dma_load_b128(i32x4 rsrc, uint32_t lds_dst, uint
 #if defined(CK_PROBE_NO_LOADS)  // measurement build only: nothing is loaded
     return;
 #endif
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen " CK_DMA_CPOL " lds"
                  :
                  : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff)
                  : "memory");
@@ -136,7 +141,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
     uint32_t nrec_a = 0, nrec_b = 0;
     // the segment being issued
     uint32_t ld_base = 0, ld_k0x2 = 0;
-    bool ld_ktail = false;
+    bool ld_ktail = false, ld_fast = false, full_tile = false;
 
     auto open_tile = [&]() __attribute__((always_inline)) {
 #if defined(CK_PROBE_SAME_TILE)  // measurement build only: every workgroup loads the operands of tile (0, 0)
@@ -150,6 +155,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         const int ra = g.M - row_a < TILE ? g.M - row_a : TILE, rb = g.N - row_b < TILE ? g.N - row_b : TILE;
         nrec_a = (uint32_t)ra * pitch32;
         nrec_b = (uint32_t)rb * pitch32;
+        full_tile = ra == TILE && rb == TILE;
         rsrc_a = make_rsrc((const char*)g.A + (int64_t)row_a * pitch32, nrec_a);
         rsrc_b = make_rsrc((const char*)g.Bt + (int64_t)row_b * pitch32, nrec_b);
     };
@@ -159,6 +165,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         ld_base = ring_base + (uint32_t)l_stage * (2 * OPB);
         ld_k0x2 = (uint32_t)l_seg * (SEGK * 2);
         ld_ktail = (l_seg + 1) * SEGK > g.K;
+        ld_fast = full_tile && !ld_ktail;
         ++opened_segs;
         if (++l_seg == nseg) { l_seg = 0; l_tc += grid; }
         if (++l_stage == S) l_stage = 0;
@@ -175,9 +182,17 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
             is_a = wave < NI;
             E = is_a ? wave : wave - NI;
         }
-        uint32_t voff = loff_w + ((uint32_t)E * load_step + ld_k0x2);
-        if (ld_ktail && (int)(ld_k0x2 >> 1) + lchunk_w * CHUNK_ELEMS >= g.K) voff = is_a ? nrec_a : nrec_b;
-        dma_load_b128(is_a ? rsrc_a : rsrc_b, ld_base + (is_a ? 0u : (uint32_t)OPB) + (uint32_t)E * 1024u, voff, 0u);
+        const uint32_t dst = ld_base + (is_a ? 0u : (uint32_t)OPB) + (uint32_t)E * 1024u;
+        const uint32_t goff = (uint32_t)E * load_step + ld_k0x2;  // scalar: row block and k offset
+        if (ld_fast) {
+            // whole tile, whole segment inside the operands: nothing can be out of range, so the
+            // scalar part rides in the (unchecked) scalar offset and no vector ALU work is needed
+            dma_load_b128(is_a ? rsrc_a : rsrc_b, dst, loff_w, goff);
+        } else {
+            uint32_t voff = loff_w + goff;
+            if (ld_ktail && (int)(ld_k0x2 >> 1) + lchunk_w * CHUNK_ELEMS >= g.K) voff = is_a ? nrec_a : nrec_b;
+            dma_load_b128(is_a ? rsrc_a : rsrc_b, dst, voff, 0u);
+        }
         ++issued_loads;
     };
 
@@ -214,6 +229,9 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
                 const int n = n_base + j * 16;
                 const int64_t off = (int64_t)m * g.N + n;
                 f32x4 v = acc[i][j] * alpha;
+#if defined(CK_PROBE_NO_EPILOGUE)  // measurement build only: nothing is written (except by a workgroup that never exists)
+                if (blockIdx.x == 0x7fffffff) *(f32x4*)(g.D + off) = v;
+#else
                 if (interior) {
                     if (beta != 0.f) v += *(const f32x4*)(g.C + off) * beta;
                     *(f32x4*)(g.D + off) = v;
@@ -227,6 +245,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
                         }
                     }
                 }
+#endif
                 acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
@@ -236,6 +255,9 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
     // outstanding (a wave's loads complete in issue order; other memory operations in flight only
     // make the wait longer, never shorter)
     auto wait_landed = [&](int X) __attribute__((always_inline)) {
+#if defined(CK_PROBE_NO_LANDING_WAIT)  // measurement build only (results are wrong): loads are never waited for
+        return;
+#endif
         const int later = issued_loads - (X + 1) * LPW;
         if (later == 2 * LPW) wait_vmcnt_imm<2 * LPW>();   // four stages in steady state
         else if (later == LPW) wait_vmcnt_imm<LPW>();      // three stages
@@ -315,7 +337,11 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
 #else
         constexpr int PER = (NF + COLS - 1) / COLS;   // fetches per column
 #endif
-        constexpr int LSTRIDE = COLS / LPK > 0 ? COLS / LPK : 1;
+#if defined(CK_FUSED_LOAD_STRIDE)
+        constexpr int LSTRIDE = CK_FUSED_LOAD_STRIDE;  // tuning builds
+#else
+        constexpr int LSTRIDE = (COLS + LPK - 1) / LPK;
+#endif
 #pragma unroll
         for (int j = PRE; j < WTC; ++j) {
             // (after the very last k-step of the stream this fetches fragments nobody uses: the

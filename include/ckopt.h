@@ -42,10 +42,13 @@ enum {
  * (wave_tile_rows*16, wave_tile_cols*16) with bar_steps_a <= C/2 and bar_steps_b <= 2, or (16, 16)
  * with bar_steps_a < wave_tile_rows and bar_steps_b < wave_tile_cols; num_producer_waves in
  * {2,4,8} (half stream A, half stream Bt) or 0 (no dedicated producers: every consumer wave also
- * streams its share of each segment; tile granularity only); num_consumer_waves in {4,8};
- * num_cus = persistent grid.
+ * streams its share of each segment and the waves meet at the workgroup barrier once per segment;
+ * tile granularity only, num_stages >= 2); num_consumer_waves in {4,8}; num_cus = persistent grid.
  * M, N need not be multiples of tile_dim and K need not be a multiple of segment_dim_k (edges are
- * zero-filled / masked), but K must be a multiple of 8 so that rows are 16-byte aligned. */
+ * zero-filled / masked). The kernels read operand rows that start on 16-byte boundaries: when K is
+ * not a multiple of 8, or A / Bt is not 16-byte aligned (2-byte alignment is required), the call
+ * first copies both operands into zero-padded rows in a stream-ordered temporary
+ * (hipMallocAsync / hipFreeAsync on `stream`, (M + N) * round_up(K, 8) * 2 bytes). */
 int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* Bt, const float* C, float* D,
                                          float alpha, float beta, int M, int N, int K, int tile_dim,
                                          int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,

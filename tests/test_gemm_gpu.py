@@ -325,3 +325,57 @@ def test_config4_long_k_shift_sync_regime(ck, oracle):
     for t in (make_tuning(ck, 128, 64, 4, 4, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 4, 2),
               make_tuning(ck, 128, 64, 4, 4, 8, "acc", 1, 3)):
         full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t, fill, rows=(0, 1024))
+
+
+# ---- K not a multiple of 8 / operands off a 16-byte boundary: zero-padded repack in front of the kernel ----
+@pytest.mark.parametrize("M,N,K", [(64, 64, 1), (130, 70, 7), (257, 129, 33), (200, 136, 1001)])
+def test_k_not_multiple_of_8_small(ck, M, N, K):
+    a = ck.fill_int(ck.DT_F16, (M, K), 61, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 61, 1, -2, 2)
+    want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)
+    for t in (make_tuning(ck, 64, 32, 3, 2, 4), make_tuning(ck, 128, 64, 2, 2, 8, "wave", 1, 1),
+              make_tuning(ck, 256, 32, 4, 0, 8), make_tuning(ck, 128, 64, 2, 4, 4, "acc", 2, 2)):
+        assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want), t
+
+
+def test_operands_off_16_byte_boundary(ck):
+    # A and Bt start 2 bytes into their allocations (K % 8 == 0): same repack path, same result
+    M, N, K = 192, 320, 256
+    a = ck.fill_int(ck.DT_F16, (M, K), 62, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 62, 1, -2, 2)
+    want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)
+    da = torch.zeros(M * K + 8, dtype=torch.float16, device="cuda")
+    db = torch.zeros(N * K + 8, dtype=torch.float16, device="cuda")
+    da[1: 1 + M * K] = torch.from_numpy(a.reshape(-1)).cuda()
+    db[3: 3 + N * K] = torch.from_numpy(bt.reshape(-1)).cuda()
+    d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    t = make_tuning(ck, 128, 64, 2, 2, 4)
+    ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, da.data_ptr() + 2, db.data_ptr() + 6, None, d, 1.0, 0.0, M, N, K,
+                                    t["tile_dim"], t["segment_dim_k"], 0, 0, t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                    t["tile_group_m"], t["num_stages"], t["num_producer_warps"], t["num_consumer_warps"],
+                                    t["num_sms"])
+    assert ck.device_status() == 0
+    assert np.array_equal(d.cpu().numpy(), want)
+
+
+def test_config5_bf16_6143x4097x3071(ck, oracle):
+    # every dimension ragged, rows of 3071 bf16 values (6142 bytes): sampled rows against the CPU
+    # oracle within the stated tolerance, and the row-sum identity over the whole result
+    M, N, K = 6143, 4097, 3071
+    fill = lambda s, shape: ck.fill_uniform(ck.DT_BF16, shape, 0xC0FFEE05, s)
+    for t in (make_tuning(ck, 256, 64, 2, 2, 8), make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 2, 1)):
+        full_size_check(ck, oracle, ck.DT_BF16, oracle.DT_BF16, M, N, K, t, fill, rows=(0, 3000, M - 8))
+    # exact at full size on small integers
+    a = ck.fill_int(ck.DT_BF16, (M, K), 0xC0FFEE05, 2, -1, 1)
+    bt = ck.fill_int(ck.DT_BF16, (N, K), 0xC0FFEE05, 3, -1, 1)
+    d = G.run_gemm(ck, ck.DT_BF16, a, bt, t=make_tuning(ck, 256, 64, 2, 2, 8))
+    ai, bi = G.as_f64(True, a).astype(np.int64), G.as_f64(True, bt).astype(np.int64)
+    assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
+    assert np.array_equal(d[M - 1], (ai[M - 1] @ bi.T).astype(np.float32))
+
+
+def test_fused_variant_full_size(ck, oracle):
+    M = N = K = 8192
+    for t in (make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 256, 32, 5, 0, 8)):
+        full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t,
+                        lambda s, shape: ck.fill_uniform(ck.DT_F16, shape, 0xC0FFEE03, s), rows=(0, 4000, 8184))

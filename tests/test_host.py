@@ -125,8 +125,8 @@ def test_launch_rejects_bad_arguments_before_touching_the_gpu(ck):
     with pytest.raises(ck.CkoptError) as e:  # beta != 0 needs C
         ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, 16, 16, None, 16, 1.0, 1.0, 256, 256, 256, **args)
     assert e.value.code == ck.ERR_NULL
-    with pytest.raises(ck.CkoptError) as e:  # misaligned A
-        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, 18, 16, None, 16, 1.0, 0.0, 256, 256, 256, **args)
+    with pytest.raises(ck.CkoptError) as e:  # A not even 2-byte aligned
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, 17, 16, None, 16, 1.0, 0.0, 256, 256, 256, **args)
     assert e.value.code == ck.ERR_ALIGNMENT
 
 
