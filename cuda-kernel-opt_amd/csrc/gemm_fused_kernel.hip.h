@@ -141,7 +141,12 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
     uint32_t nrec_a = 0, nrec_b = 0;
     // the segment being issued
     uint32_t ld_base = 0, ld_k0x2 = 0;
-    bool ld_ktail = false, ld_fast = false, full_tile = false;
+    bool ld_ktail = false, full_tile = false;
+    int ld_mode = 0;                      // 0: no segment open, 1: fast form, 2: slow form
+    uint32_t ld_dst_w = 0, ld_goff_w = 0;  // fast form: LDS address and global offset of this wave's load 0
+    uint32_t goff_step[HALF];              // global offset of load ii relative to load 0
+#pragma unroll
+    for (int ii = 0; ii < HALF; ++ii) goff_step[ii] = (uint32_t)(ii * CW) * load_step;
 
     auto open_tile = [&]() __attribute__((always_inline)) {
 #if defined(CK_PROBE_SAME_TILE)  // measurement build only: every workgroup loads the operands of tile (0, 0)
@@ -165,35 +170,41 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         ld_base = ring_base + (uint32_t)l_stage * (2 * OPB);
         ld_k0x2 = (uint32_t)l_seg * (SEGK * 2);
         ld_ktail = (l_seg + 1) * SEGK > g.K;
-        ld_fast = full_tile && !ld_ktail;
+        ld_mode = STATIC_SPLIT && full_tile && !ld_ktail ? 1 : 2;
+        ld_dst_w = ld_base + (uint32_t)wave * 1024u;
+        ld_goff_w = (uint32_t)wave * load_step + ld_k0x2;
         ++opened_segs;
         if (++l_seg == nseg) { l_seg = 0; l_tc += grid; }
         if (++l_stage == S) l_stage = 0;
     };
-    // load i (0 .. LPW-1) of the open segment. The whole global offset goes through the range-checked
-    // vector offset: rows past the tile edge and k past K land outside the descriptor and read as zero.
+    // load i (0 .. LPW-1) of the open segment. Fast form (whole tile, whole segment inside the
+    // operands, nothing can be out of range): the per-lane offset is a constant of the wave and
+    // everything else is scalar - M0 and the (unchecked) scalar offset, one add each. Slow form (edge
+    // tiles, K tail): the whole global offset goes through the range-checked vector offset, so rows
+    // past the tile edge and k past K land outside the descriptor and read as zero.
     auto issue_load = [&](int i) __attribute__((always_inline)) {
         bool is_a;
-        int E;
+        int E, ii;
         if (STATIC_SPLIT) {
             is_a = i < HALF;
-            E = wave + (i % HALF) * CW;
+            ii = i % HALF;
+            E = wave + ii * CW;
         } else {
             is_a = wave < NI;
+            ii = 0;
             E = is_a ? wave : wave - NI;
         }
-        const uint32_t dst = ld_base + (is_a ? 0u : (uint32_t)OPB) + (uint32_t)E * 1024u;
-        const uint32_t goff = (uint32_t)E * load_step + ld_k0x2;  // scalar: row block and k offset
-        if (ld_fast) {
-            // whole tile, whole segment inside the operands: nothing can be out of range, so the
-            // scalar part rides in the (unchecked) scalar offset and no vector ALU work is needed
-            dma_load_b128(is_a ? rsrc_a : rsrc_b, dst, loff_w, goff);
-        } else {
-            uint32_t voff = loff_w + goff;
+        if (ld_mode == 1) {
+            dma_load_b128(is_a ? rsrc_a : rsrc_b, ld_dst_w + (is_a ? 0u : (uint32_t)OPB) + (uint32_t)(ii * CW) * 1024u, loff_w,
+                          ld_goff_w + goff_step[ii]);
+            ++issued_loads;
+        } else if (ld_mode == 2) {
+            const uint32_t dst = ld_base + (is_a ? 0u : (uint32_t)OPB) + (uint32_t)E * 1024u;
+            uint32_t voff = loff_w + ((uint32_t)E * load_step + ld_k0x2);
             if (ld_ktail && (int)(ld_k0x2 >> 1) + lchunk_w * CHUNK_ELEMS >= g.K) voff = is_a ? nrec_a : nrec_b;
             dma_load_b128(is_a ? rsrc_a : rsrc_b, dst, voff, 0u);
+            ++issued_loads;
         }
-        ++issued_loads;
     };
 
     // ---- multiplier side -------------------------------------------------------------------------------
@@ -258,6 +269,10 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
 #if defined(CK_PROBE_NO_LANDING_WAIT)  // measurement build only (results are wrong): loads are never waited for
         return;
 #endif
+#if defined(CK_PROBE_WAIT0)  // measurement build only: always drain (what two stages need), no ladder
+        wait_vmcnt_imm<0>();
+        return;
+#endif
         const int later = issued_loads - (X + 1) * LPW;
         if (later == 2 * LPW) wait_vmcnt_imm<2 * LPW>();   // four stages in steady state
         else if (later == LPW) wait_vmcnt_imm<LPW>();      // three stages
@@ -292,6 +307,11 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         const uint32_t pb_k = (st + b_lane) ^ (uint32_t)((last_ks ? 0 : KS + 1) * 64);
 
         if (last_ks) {
+            // The next segment's parameters are worked out here, ahead of the waits: behind the barrier
+            // nothing but the loads themselves stands between the waves and their MFMAs. (All chunks of
+            // the previous segment were issued by the k-step before this one.)
+            ld_mode = 0;
+            if (has_next_seg && opened_segs < total_segs) open_segment();
             CK_T0();
             // The last fragments of this segment must be in registers before the barrier releases
             // their stage. The wait is requested through a use of the registers the compiler can
@@ -311,20 +331,10 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         // chunk of LPK loads this k-step issues: at a segment's last k-step (behind the barrier) chunk 0
         // of the segment that goes into the stage just released, otherwise the next chunk of the
         // segment opened at the previous segment's last k-step
-        bool loading;
-        if (last_ks) {
-            loading = false;
-            if (has_next_seg) {
-                CK_T0();
-                wg_barrier();
-                CK_T1(t_bar);
-                if (opened_segs < total_segs) {
-                    open_segment();
-                    loading = true;
-                }
-            }
-        } else {
-            loading = issued_loads < opened_segs * LPW;
+        if (last_ks && has_next_seg) {
+            CK_T0();
+            wg_barrier();
+            CK_T1(t_bar);
         }
         constexpr int CHUNK = last_ks ? 0 : KS + 1;
         __builtin_amdgcn_sched_barrier(0);
@@ -355,12 +365,10 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
 #endif
             }
             __builtin_amdgcn_sched_barrier(0);
-            if (loading) {
 #pragma unroll
-                for (int l = 0; l < LPK; ++l) {
-                    const int col = l * LSTRIDE < COLS ? l * LSTRIDE : COLS - 1;
-                    if (col == j - PRE) issue_load(CHUNK * LPK + l);
-                }
+            for (int l = 0; l < LPK; ++l) {
+                const int col = l * LSTRIDE < COLS ? l * LSTRIDE : COLS - 1;
+                if (col == j - PRE) issue_load(CHUNK * LPK + l);
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -385,6 +393,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
 #pragma unroll
             for (int i = 0; i < LPW; ++i) issue_load(i);
         }
+        ld_mode = 0;  // everything opened so far is issued
         wait_landed(0);
         wg_barrier();
         {
