@@ -78,8 +78,8 @@ def cpu_baseline(ck, kind, dtype, a, b, M, N, K, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="config3_fp16_8192", choices=sorted(WORKLOADS))
     # tuning flags default to the best measured tuple of the workload (TUNED below)
     ap.add_argument("--tile", type=int, default=None)
@@ -97,6 +97,10 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device copy kernel (reads 1 GiB, writes 1 GiB): the reference "
                          "reading for FETCH_SIZE / WRITE_SIZE counter runs")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="run only the bare inner-loop probe (ckopt_probe_mfma_ceiling): what the device sustains with "
+                         "constant / random operands, without / with the direct-to-LDS loads")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the bare inner-loop probe of the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
     args = ap.parse_args()
@@ -115,6 +119,15 @@ def main():
     ck = load_package()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.ceiling:
+        res = {}
+        for rnd in (0, 1):
+            for loads in (0, 1):
+                key = "%s_operands_%s" % ("random" if rnd else "constant", "with_loads" if loads else "no_loads")
+                res[key] = round(ck.probe_mfma_ceiling(rnd, loads, 400000), 1)
+        print(json.dumps({"probe": "bare inner loop of the 256x256 tile GEMM, 8 waves per CU, ~0.2 s per case",
+                          "unit": "TFLOP/s", "nominal_peak": PEAK_TFLOPS["mfma_f16"], **res}))
+        return 0
     if args.calibrate_copy:
         n = 1 << 28  # fp32 elements: 1 GiB
         src = torch.ones(n, dtype=torch.float32, device=dev)
@@ -235,6 +248,13 @@ def main():
                      "unit": "TFLOP/s", "frac": round(achieved / peak, 4), "traffic": traffic,
                      "kernel_ms": round(kern_ms, 5), "flops_per_launch": flops},
     }
+    if kind == "gemm" and args.workload == "config3_fp16_8192" and not args.no_ceiling:
+        # what the bare inner loop of this tile shape sustains on this device with random operands and the
+        # loads of the real data flow (no synchronisation, no waiting, no epilogue): the device's power limit
+        # keeps it well below the nominal peak, and no kernel of this shape can exceed it
+        ceil = ck.probe_mfma_ceiling(1, 1, 400000)
+        out["roofline"]["measured_ceiling"] = round(ceil, 1)
+        out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
     if check is not None:
         out["parity_check"] = check
     if not args.no_cpu_baseline:

@@ -1,0 +1,156 @@
+// Measurement kernel, no counterpart in the reference: the inner loop of the 256 x 256 tile GEMM with
+// everything removed that a real GEMM adds on top - no flags, no barrier, no waiting for data, no
+// epilogue. Eight waves per CU; per wave and k-step 32 MFMAs (16x16x32 f16) on fragments fetched from
+// LDS one k-step ahead (12 ds_read_b128 at the fragment addresses of the seg_k 64 ring), optionally
+// four direct-to-LDS loads of 8 rows x 128 bytes that stream through an L2-resident window. What it
+// sustains is the ceiling a kernel of this shape can reach on the device at hand: with constant
+// operand values the matrix cores run near their nominal rate, with random operand values the
+// device's power limit lowers the clock well below it.
+#include <hip/hip_runtime.h>
+
+#include <stdint.h>
+
+#include "ck_common.h"
+
+namespace {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+#define CKP_LDS __attribute__((address_space(3)))
+
+constexpr int PROBE_LDS_BYTES = 128 * 1024;
+constexpr uint32_t WINDOW_BYTES = 512u * 1024u;  // per workgroup class; 4 classes per XCD stay L2 resident
+constexpr int WINDOW_CLASSES = 32;
+
+__device__ __forceinline__ void probe_dma_b128(i32x4 rsrc, uint32_t lds_dst, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+
+template <bool RANDOM, bool LOADS>
+__global__ __launch_bounds__(512) void ceiling_probe_kernel(const char* window, int ksteps, float* sink) {
+    extern __shared__ __attribute__((aligned(1024))) char probe_smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(CKP_LDS char*)probe_smem;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    // the first 64 KiB play the ring stage the fragments come from, the second 64 KiB receive the loads
+    for (int i = threadIdx.x; i < PROBE_LDS_BYTES / 4; i += 512) {
+        uint32_t v = 0x3c003c00u;  // two fp16 ones
+        if (RANDOM) {
+            uint32_t h = (uint32_t)i * 2654435761u + blockIdx.x * 40503u;
+            h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+            // two fp16 values of random sign and mantissa, magnitude 2^-5 .. 2^-1
+            v = ((h & 0x83ffu) | ((10u + ((h >> 10) & 3u)) << 10)) | ((((h >> 16) & 0x83ffu) | ((10u + ((h >> 26) & 3u)) << 10)) << 16);
+        }
+        ((CKP_LDS uint32_t*)probe_smem)[i] = v;
+    }
+    const uint64_t p = (uint64_t)(uintptr_t)(window + (size_t)(blockIdx.x % WINDOW_CLASSES) * WINDOW_BYTES);
+    i32x4 rsrc;
+    rsrc[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    rsrc[1] = __builtin_amdgcn_readfirstlane((int)((p >> 32) & 0xffffu));
+    rsrc[2] = (int)WINDOW_BYTES;
+    rsrc[3] = 0x00020000;
+    // 8 rows x 128 bytes per wave load, rows 16 KiB apart (the pitch of a K = 8192 fp16 operand)
+    const uint32_t voff = (uint32_t)(lane / 8) * 16384u + (uint32_t)(lane % 8) * 16u;
+    const int lr = lane & 15, lg = lane >> 4, key = (lr >> 1) % 8;
+    const uint32_t a_lane = lds0 + (uint32_t)((wave / 2) * 64 + lr) * 128u + (uint32_t)((lg ^ key) * 16);
+    const uint32_t b_lane = lds0 + 32768u + (uint32_t)((wave % 2) * 128 + lr) * 128u + (uint32_t)((lg ^ key) * 16);
+    u32x4 fr[2][12];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+        fr[0][i] = u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+        fr[1][i] = fr[0][i];
+    }
+    f32x4 acc[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+    uint32_t gpos = 0;
+    for (int it = 0; it < ksteps; it += 2) {
+#pragma unroll
+        for (int P = 0; P < 2; ++P) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int f = j * 2 + q;
+                    if (f < 4) fr[1 - P][f] = *(const CKP_LDS u32x4*)(uintptr_t)((a_lane ^ (uint32_t)(P * 64)) + f * 2048);
+                    else if (f < 12) fr[1 - P][f] = *(const CKP_LDS u32x4*)(uintptr_t)((b_lane ^ (uint32_t)(P * 64)) + (f - 4) * 2048);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (LOADS && j % 2 == 0) {
+                    // distinct lines per wave and load; the window (4 row groups x 16 KiB of k) wraps
+                    const int d = j / 2;
+                    probe_dma_b128(rsrc, lds0 + 65536u + (uint32_t)(wave * 4 + d) * 1024u, voff,
+                                   ((gpos + (uint32_t)(wave * 4 + d) * 128u) & 0x3fffu) + ((gpos >> 14) & 3u) * 131072u);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fr[P][4 + j]), __builtin_bit_cast(f16x8, fr[P][i]), acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (LOADS) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            gpos += 8u * 4u * 128u;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += acc[i][j][0] + acc[i][j][3];
+    sink[blockIdx.x * 512 + threadIdx.x] = s;
+}
+
+template <bool RANDOM, bool LOADS>
+hipError_t launch_probe(int cus, const char* window, int ksteps, float* sink, hipStream_t s) {
+    auto kern = ceiling_probe_kernel<RANDOM, LOADS>;
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, ck::LDS_BYTES_PER_CU);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(cus), dim3(512), PROBE_LDS_BYTES, s, window, ksteps, sink);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out) {
+    using namespace ck;
+    if (!tflops_out || ksteps < 2 || ksteps > (1 << 26)) return CK_ERR_BAD_PARAM;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return CK_ERR_HIP;
+    // the last load of a window reaches 7 rows x 16 KiB + 3 row groups x 128 KiB + 16 KiB past its start
+    const size_t window_bytes = (size_t)WINDOW_CLASSES * WINDOW_BYTES + (1u << 20);
+    char* window = nullptr;
+    float* sink = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int rc = CK_ERR_HIP;
+    do {
+        if (hipMalloc((void**)&window, window_bytes) != hipSuccess) break;
+        if (hipMalloc((void**)&sink, (size_t)cus * 512 * sizeof(float)) != hipSuccess) break;
+        if (hipMemset(window, 0, window_bytes) != hipSuccess) break;
+        if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) break;
+        auto go = [&](int n) {
+            if (random_operands) return with_loads ? launch_probe<true, true>(cus, window, n, sink, nullptr) : launch_probe<true, false>(cus, window, n, sink, nullptr);
+            return with_loads ? launch_probe<false, true>(cus, window, n, sink, nullptr) : launch_probe<false, false>(cus, window, n, sink, nullptr);
+        };
+        if (go(ksteps / 8 + 2) != hipSuccess) break;   // warm-up
+        if (hipEventRecord(e0, nullptr) != hipSuccess) break;
+        if (go(ksteps) != hipSuccess) break;
+        if (hipEventRecord(e1, nullptr) != hipSuccess || hipEventSynchronize(e1) != hipSuccess) break;
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess || ms <= 0.f) break;
+        const int n = (ksteps + 1) / 2 * 2;
+        // per CU and k-step: 8 waves x 32 MFMAs x 16*16*32*2 flop = a 256 x 256 x 32 block
+        *tflops_out = (double)cus * n * 8.0 * 32.0 * 16384.0 / (ms * 1e-3) * 1e-12;
+        rc = CK_OK;
+    } while (false);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (window) (void)hipFree(window);
+    if (sink) (void)hipFree(sink);
+    return rc;
+}

@@ -119,6 +119,17 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  * flag waits (lo, hi), wait calls, polls, read-ahead hits. All zero in the normal build. */
 int ckopt_probe_counters(void* stream, unsigned int* out, int nwords);
 
+/* Measures what the inner loop of the 256 x 256 tile GEMM sustains on the current device when nothing
+ * of a real GEMM is in its way (no synchronisation, no waiting for data, no epilogue): 8 waves per CU,
+ * per wave and k-step 32 MFMAs on fragments read from LDS one k-step ahead, with with_loads != 0 also
+ * the four direct-to-LDS loads per wave and k-step of the real data flow (from an L2-resident
+ * window). random_operands selects random instead of constant fragment values: the power the matrix
+ * cores draw, and with it the clock the device sustains, depends on the operand values. Runs ksteps
+ * k-steps per wave on every CU (after a warm-up), allocates and frees its own buffers, synchronises,
+ * and returns the rate in TFLOP/s: the practical ceiling next to the nominal peak. No reference
+ * counterpart. */
+int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out);
+
 /* Process-wide tuning switches that are not launcher parameters in the reference:
  * key 0: LDS XOR swizzle on/off (default 1); key 1: spin limit of bounded waits (default 1<<22);
  * key 2: number of XCDs assumed by the workgroup->tile remap (default 8; 1 disables the remap).

@@ -379,3 +379,11 @@ def test_fused_variant_full_size(ck, oracle):
     for t in (make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 256, 32, 5, 0, 8)):
         full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t,
                         lambda s, shape: ck.fill_uniform(ck.DT_F16, shape, 0xC0FFEE03, s), rows=(0, 4000, 8184))
+
+
+def test_inner_loop_ceiling_probe_runs(ck):
+    # measurement helper: finite positive rates, and the loads never make the bare loop faster
+    r = {(rnd, ld): ck.probe_mfma_ceiling(rnd, ld, 20000) for rnd in (0, 1) for ld in (0, 1)}
+    assert all(np.isfinite(v) and 50.0 < v < 2600.0 for v in r.values()), r
+    with pytest.raises(ck.CkoptError):
+        ck.probe_mfma_ceiling(0, 0, 1)
