@@ -1,0 +1,99 @@
+// C++ face of libckopt.so: the reference's launcher templates, same names and parameter order, as thin
+// wrappers over the C ABI of ckopt.h. A failed call throws ckopt::Error where the reference asserts.
+//
+//   gemm_shmem_tc_async_opt_port<DT,DT_ACC>   matmul_shmem_tc_async_opt_port_2.cu:1088-1109 (port_1:889-908 and
+//                                             port_0:515-532 are the overloads with fewer parameters)
+//   matmul_shmem<DT,DT_ACC>                   matmul_shmem.cu:143-152
+//   get_shmem_req<DT,DT_ACC>                  port_2.cu:1057-1066        get_num_acc / get_warp_tile_rows  :158-169
+//
+// DT is one of ckopt::half_t (IEEE fp16; layout-compatible with __half), ckopt::bfloat16_t, float, int;
+// DT_ACC is float (GEMM) or equals DT (matmul_shmem). Pointers are device memory owned by the caller.
+#ifndef CKOPT_HPP
+#define CKOPT_HPP
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+
+#include "ckopt.h"
+
+namespace ckopt {
+
+using half_t = _Float16;
+struct bfloat16_t { std::uint16_t bits; };
+
+struct Error : std::runtime_error {
+    int code;
+    Error(int c, const char* where) : std::runtime_error(std::string(where) + ": " + ckopt_error_string(c)), code(c) {}
+};
+inline void check(int rc, const char* where) { if (rc != CKOPT_OK) throw Error(rc, where); }
+
+template <typename DT> struct dtype_of;
+template <> struct dtype_of<half_t> { static constexpr int value = CKOPT_DT_F16; };
+template <> struct dtype_of<bfloat16_t> { static constexpr int value = CKOPT_DT_BF16; };
+template <> struct dtype_of<float> { static constexpr int value = CKOPT_DT_F32; };
+template <> struct dtype_of<int> { static constexpr int value = CKOPT_DT_I32; };
+
+// port_2: individually signalled upper-left units (bar_steps) + granularity (bar_step_rows)
+template <typename DT, typename DT_ACC>
+void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B /* transposed: N x K */, const DT_ACC* C, DT_ACC* D, DT_ACC alpha,
+                                  DT_ACC beta, int M, int N, int K, int tile_dim, int segment_dim_k, int bar_steps_a,
+                                  int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
+                                  int num_producer_warps, int num_consumer_warps, int num_sms, void* stream = nullptr) {
+    static_assert(std::is_same<DT_ACC, float>::value, "fp32 accumulate/output");
+    check(ckopt_gemm_shmem_tc_async_opt_port_2(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
+                                               bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m,
+                                               num_stages, num_producer_warps, num_consumer_warps, num_sms, stream),
+          "gemm_shmem_tc_async_opt_port");
+}
+// port_1: granularity only
+template <typename DT, typename DT_ACC>
+void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B, const DT_ACC* C, DT_ACC* D, DT_ACC alpha, DT_ACC beta, int M, int N,
+                                  int K, int tile_dim, int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
+                                  int tile_group_m, int num_stages, int num_producer_warps, int num_consumer_warps, int num_sms,
+                                  void* stream = nullptr) {
+    static_assert(std::is_same<DT_ACC, float>::value, "fp32 accumulate/output");
+    check(ckopt_gemm_shmem_tc_async_opt_port_1(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
+                                               bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+                                               num_consumer_warps, num_sms, stream),
+          "gemm_shmem_tc_async_opt_port (port_1)");
+}
+// port_0: one signal pair per stage
+template <typename DT, typename DT_ACC>
+void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B, const DT_ACC* C, DT_ACC* D, DT_ACC alpha, DT_ACC beta, int M, int N,
+                                  int K, int tile_dim, int segment_dim_k, int tile_group_m, int num_stages,
+                                  int num_producer_warps, int num_consumer_warps, int num_sms, void* stream = nullptr) {
+    static_assert(std::is_same<DT_ACC, float>::value, "fp32 accumulate/output");
+    check(ckopt_gemm_shmem_tc_async_opt_port_0(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
+                                               tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, stream),
+          "gemm_shmem_tc_async_opt_port (port_0)");
+}
+
+template <typename DT, typename DT_ACC>
+void matmul_shmem(const DT* A, const DT* B, DT* C, int M, int N, int K, int tile_dim, int block_rows, bool b_transposed = false,
+                  void* stream = nullptr) {
+    check(ckopt_matmul_shmem(dtype_of<DT>::value, A, B, C, M, N, K, tile_dim, block_rows, b_transposed ? 1 : 0, stream), "matmul_shmem");
+}
+
+template <typename DT, typename DT_ACC>
+int get_shmem_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b,
+                  int num_stages, int num_consumer_warps) {
+    const int r = ckopt_get_lds_req(tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, num_stages,
+                                    num_consumer_warps);
+    if (r < 0) throw Error(r, "get_shmem_req");
+    return r;
+}
+inline int get_num_acc(int tile_dim, int num_consumer_warps) {
+    const int r = ckopt_get_num_acc(tile_dim, num_consumer_warps);
+    if (r < 0) throw Error(r, "get_num_acc");
+    return r;
+}
+inline int get_warp_tile_rows(int tile_dim, int num_consumer_warps) {
+    const int r = ckopt_get_warp_tile_rows(tile_dim, num_consumer_warps);
+    if (r < 0) throw Error(r, "get_warp_tile_rows");
+    return r;
+}
+
+}  // namespace ckopt
+#endif  // CKOPT_HPP

@@ -1,0 +1,182 @@
+// Test driver in the role of the reference's per-file main() (matmul_shmem_tc_async_opt_port_2.cu:1171-1566) and
+// its fixtures (matmul_test.h): constant-matrix correctness sweep, random accuracy counts against the CPU
+// oracle, and a performance sweep that prints the reference's tuple-per-line format
+//   (tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m,
+//    num_stages, num_producer_warps, num_consumer_warps): TFLOP/s
+// Everything goes through the launcher templates of include/ckopt.hpp, i.e. through the C ABI. Test
+// infrastructure: it links the CPU oracle for the accuracy check.
+//
+//   gemm_driver correctness | accuracy | performance [dim] | all
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "ckopt.hpp"
+
+extern "C" {
+int oracle_gemm_blocked(int dtype, const uint16_t* a, const uint16_t* bt, const float* c, float* out, float alpha, float beta,
+                        int M, int N, int K, int row0, int row1, int threads);
+int64_t oracle_count_incorrect(const float* expected, const float* res, int64_t n, float atol);
+}
+
+#define HIP_OK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { std::fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_)); std::exit(2); } } while (0)
+
+using DT = ckopt::half_t;
+using DT_ACC = float;
+
+struct Tuple { int tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, rows_a, rows_b, tile_group_m, num_stages, producers, consumers; };
+
+static void print_tuple(const Tuple& t) {
+    std::printf("(%d, %d, %d, %d, %d, %d, %d, %d, %d, %d)", t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b, t.rows_a, t.rows_b,
+                t.tile_group_m, t.num_stages, t.producers, t.consumers);
+}
+
+// every legal tuple of a small grid of knobs, all three granularities with all their bar_steps
+static std::vector<Tuple> tuples(int stride) {
+    std::vector<Tuple> out;
+    int n = 0;
+    const int tiles[] = {64, 128, 256}, cons[] = {4, 8}, segs[] = {32, 64, 128}, prods[] = {0, 2, 4};
+    for (int tile : tiles) for (int c : cons) {
+        if (ckopt_get_num_acc(tile, c) < 0 || ckopt_get_num_acc(tile, c) > 32) continue;
+        const int wtr = ckopt::get_warp_tile_rows(tile, c), wtc = ckopt::get_num_acc(tile, c) / wtr;
+        const int rows_a[3] = {16, wtr * 16, tile}, rows_b[3] = {16, wtc * 16, tile};
+        const int sa_end[3] = {wtr - 1, c / 2, 0}, sb_end[3] = {wtc - 1, 2, 0};
+        for (int sk : segs) for (int stages = 1; stages <= 4; ++stages) for (int p : prods) for (int g = 0; g < 3; ++g)
+            for (int sa = 0; sa <= sa_end[g]; ++sa) for (int sb = 0; sb <= sb_end[g]; ++sb) {
+                const Tuple t{tile, sk, sa, sb, rows_a[g], rows_b[g], 1 + (n % 5), stages, p, c};
+                if (ckopt_check_gemm_tuning(tile, sk, sa, sb, t.rows_a, t.rows_b, t.tile_group_m, stages, p, c, 256) != CKOPT_OK) continue;
+                if (n++ % stride == 0) out.push_back(t);
+            }
+    }
+    return out;
+}
+
+struct Device {
+    DT *A = nullptr, *B = nullptr;
+    DT_ACC *C = nullptr, *D = nullptr;
+    size_t n;
+    explicit Device(size_t elems) : n(elems) {
+        HIP_OK(hipMalloc((void**)&A, n * sizeof(DT))); HIP_OK(hipMalloc((void**)&B, n * sizeof(DT)));
+        HIP_OK(hipMalloc((void**)&C, n * sizeof(DT_ACC))); HIP_OK(hipMalloc((void**)&D, n * sizeof(DT_ACC)));
+    }
+    ~Device() { (void)hipFree(A); (void)hipFree(B); (void)hipFree(C); (void)hipFree(D); }
+};
+
+static void launch(const Device& d, float alpha, float beta, int dim, const Tuple& t, int cus) {
+    ckopt::gemm_shmem_tc_async_opt_port<DT, DT_ACC>(d.A, d.B, d.C, d.D, alpha, beta, dim, dim, dim, t.tile_dim, t.segment_dim_k, t.bar_steps_a,
+                                                     t.bar_steps_b, t.rows_a, t.rows_b, t.tile_group_m, t.num_stages, t.producers, t.consumers, cus);
+}
+
+// A = 1, B = 10, C = 1: every element of D is alpha * 10 * dim + beta (the reference's closed form)
+static int correctness(int cus) {
+    const int dim_max = 1024;
+    const size_t n = (size_t)dim_max * dim_max;
+    std::vector<DT> a(n), b(n);
+    std::vector<DT_ACC> c(n), res(n);
+    ckopt::check(ckopt_fill_constant(CKOPT_DT_F16, a.data(), (int64_t)n, 1.f), "fill");
+    ckopt::check(ckopt_fill_constant(CKOPT_DT_F16, b.data(), (int64_t)n, 10.f), "fill");
+    ckopt::check(ckopt_fill_constant(CKOPT_DT_F32, c.data(), (int64_t)n, 1.f), "fill");
+    Device d(n);
+    HIP_OK(hipMemcpy(d.A, a.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.B, b.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.C, c.data(), n * sizeof(DT_ACC), hipMemcpyHostToDevice));
+    int failed = 0, run = 0;
+    unsigned lcg = 12345u;
+    for (const Tuple& t : tuples(7)) {
+        lcg = lcg * 1664525u + 1013904223u;
+        const int dim = (run % 4 == 0) ? dim_max : std::max(t.tile_dim, (int)((lcg >> 8) % (dim_max + 1)) / t.tile_dim * t.tile_dim);
+        HIP_OK(hipMemset(d.D, 0, n * sizeof(DT_ACC)));
+        launch(d, 1.f, 1.f, dim, t, cus);
+        HIP_OK(hipMemcpy(res.data(), d.D, n * sizeof(DT_ACC), hipMemcpyDeviceToHost));
+        const float want = 10.f * dim + 1.f;
+        bool ok = ckopt_device_status(nullptr) == 0;
+        for (size_t i = 0; ok && i < (size_t)dim * dim; ++i) ok = std::fabs(res[i] - want) <= 0.001f;
+        for (size_t i = (size_t)dim * dim; ok && i < n; ++i) ok = res[i] == 0.f;
+        ++run;
+        if (!ok) { ++failed; std::printf("FAILED dim %d ", dim); print_tuple(t); std::printf("\n"); }
+    }
+    std::printf("correctness: %d tuples, %d failed\n", run, failed);
+    return failed;
+}
+
+// uniform[-1,1) operands; number of elements with |cpu - gpu| > 0.1 (the reference's accuracy count) must be 0
+static int accuracy(int cus) {
+    const int dim = 512;
+    const size_t n = (size_t)dim * dim;
+    std::vector<DT> a(n), b(n);
+    std::vector<DT_ACC> c(n), res(n), ref(n);
+    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F16, a.data(), (int64_t)n, 77, 0, -1.f, 1.f), "fill");
+    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F16, b.data(), (int64_t)n, 77, 1, -1.f, 1.f), "fill");
+    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F32, c.data(), (int64_t)n, 77, 2, -1.f, 1.f), "fill");
+    if (oracle_gemm_blocked(0, (const uint16_t*)a.data(), (const uint16_t*)b.data(), c.data(), ref.data(), 1.f, 1.f, dim, dim, dim, 0, dim, 0) != 0) return 1;
+    Device d(n);
+    HIP_OK(hipMemcpy(d.A, a.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.B, b.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.C, c.data(), n * sizeof(DT_ACC), hipMemcpyHostToDevice));
+    int failed = 0, run = 0;
+    for (const Tuple& t : tuples(23)) {
+        HIP_OK(hipMemset(d.D, 0, n * sizeof(DT_ACC)));
+        launch(d, 1.f, 1.f, dim, t, cus);
+        HIP_OK(hipMemcpy(res.data(), d.D, n * sizeof(DT_ACC), hipMemcpyDeviceToHost));
+        const long long bad = (long long)oracle_count_incorrect(ref.data(), res.data(), (int64_t)n, 0.1f);
+        ++run;
+        if (bad != 0 || ckopt_device_status(nullptr) != 0) { ++failed; print_tuple(t); std::printf(": %lld incorrect\n", bad); }
+    }
+    std::printf("accuracy: %d tuples at %d^3, %d with incorrect elements\n", run, dim, failed);
+    return failed;
+}
+
+static int performance(int dim, int cus) {
+    const size_t n = (size_t)dim * dim;
+    std::vector<DT> a(n), b(n);
+    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F16, a.data(), (int64_t)n, 78, 0, -1.f, 1.f), "fill");
+    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F16, b.data(), (int64_t)n, 78, 1, -1.f, 1.f), "fill");
+    Device d(n);
+    HIP_OK(hipMemcpy(d.A, a.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.B, b.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    HIP_OK(hipMemset(d.C, 0, n * sizeof(DT_ACC)));
+    hipEvent_t start, stop;
+    HIP_OK(hipEventCreate(&start)); HIP_OK(hipEventCreate(&stop));
+    const int num_reps = 20;
+    const Tuple sweep[] = {{256, 64, 0, 0, 256, 256, 4, 2, 2, 8}, {256, 64, 0, 0, 256, 256, 4, 2, 0, 8}, {256, 32, 0, 0, 256, 256, 4, 4, 4, 8},
+                           {256, 32, 0, 0, 256, 256, 4, 5, 0, 8}, {256, 64, 2, 1, 64, 128, 4, 2, 2, 8}, {128, 64, 0, 0, 128, 128, 4, 4, 2, 8},
+                           {128, 64, 2, 2, 32, 64, 4, 4, 4, 8}, {128, 64, 1, 3, 16, 16, 4, 4, 4, 8}, {128, 128, 0, 0, 128, 128, 4, 2, 0, 8},
+                           {64, 64, 0, 0, 64, 64, 4, 4, 2, 4}};
+    for (const Tuple& t : sweep) {
+        if (ckopt_check_gemm_tuning(t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b, t.rows_a, t.rows_b, t.tile_group_m, t.num_stages,
+                                    t.producers, t.consumers, cus) != CKOPT_OK) continue;
+        launch(d, 1.f, 0.f, dim, t, cus);
+        HIP_OK(hipEventRecord(start, nullptr));
+        for (int j = 0; j < num_reps; ++j) launch(d, 1.f, 0.f, dim, t, cus);
+        HIP_OK(hipEventRecord(stop, nullptr));
+        HIP_OK(hipEventSynchronize(stop));
+        float ms = 0.f;
+        HIP_OK(hipEventElapsedTime(&ms, start, stop));
+        print_tuple(t);
+        std::printf(": %.2f\n", 2.0 * dim * dim * 1e-9 * dim * num_reps / ms);
+    }
+    const int st = ckopt_device_status(nullptr);
+    HIP_OK(hipEventDestroy(start)); HIP_OK(hipEventDestroy(stop));
+    return st != 0;
+}
+
+int main(int argc, char** argv) {
+    const char* what = argc > 1 ? argv[1] : "all";
+    int cus = 0;
+    HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, 0));
+    int failed = 0;
+    try {
+        if (!std::strcmp(what, "correctness") || !std::strcmp(what, "all")) failed += correctness(cus);
+        if (!std::strcmp(what, "accuracy") || !std::strcmp(what, "all")) failed += accuracy(cus);
+        if (!std::strcmp(what, "performance") || !std::strcmp(what, "all")) failed += performance(argc > 2 ? std::atoi(argv[2]) : 4096, cus);
+    } catch (const ckopt::Error& e) {
+        std::fprintf(stderr, "%s (code %d)\n", e.what(), e.code);
+        return 3;
+    }
+    std::printf(failed ? "FAILED\n" : "PASSED\n");
+    return failed ? 1 : 0;
+}

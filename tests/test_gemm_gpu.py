@@ -387,3 +387,17 @@ def test_inner_loop_ceiling_probe_runs(ck):
     assert all(np.isfinite(v) and 50.0 < v < 2600.0 for v in r.values()), r
     with pytest.raises(ck.CkoptError):
         ck.probe_mfma_ceiling(0, 0, 1)
+
+
+def test_cpp_driver_through_the_launcher_templates(ck):
+    # the C++ face (include/ckopt.hpp: the reference's launcher templates over the C ABI) driven by a test
+    # main in the role of the reference's own: constant-matrix sweep, accuracy counts, tuple-per-line timing
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "build", "gemm_driver")
+    assert os.path.exists(exe), "tests/cpp/build/gemm_driver is not built (make -C tests/cpp)"
+    r = subprocess.run([exe, "all", "2048"], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "PASSED" in r.stdout and "correctness:" in r.stdout and "accuracy:" in r.stdout
+    lines = [l for l in r.stdout.splitlines() if l.startswith("(") and "): " in l]
+    assert len(lines) >= 8 and all(float(l.split("): ")[1]) > 1.0 for l in lines)
