@@ -27,6 +27,8 @@ WORKLOADS = {
     "config3_fp16_8192": ("gemm", "f16", 8192, 8192, 8192, "uniform"),
     "config4_fp16_2048x2048x32768": ("gemm", "f16", 2048, 2048, 32768, "normal"),
     "config5_bf16_6143x4097x3071": ("gemm", "bf16", 6143, 4097, 3071, "uniform"),
+    # not a BASELINE config: the size the reference's own performance driver times (port_2.cu:1554-1556)
+    "config6_fp16_16384": ("gemm", "f16", 16384, 16384, 16384, "uniform"),
 }
 
 
@@ -36,6 +38,7 @@ TUNED = {
     "config3_fp16_8192": (256, 64, 2, 2, 8),
     "config4_fp16_2048x2048x32768": (128, 128, 2, 0, 8),
     "config5_bf16_6143x4097x3071": (256, 64, 2, 2, 8),
+    "config6_fp16_16384": (256, 64, 2, 2, 8),
 }
 
 
