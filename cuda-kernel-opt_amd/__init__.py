@@ -28,6 +28,8 @@ _i, _f, _p, _i64, _u64 = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c
 
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2_lp.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2_lp.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_1.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_1.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 12 + [_p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_0.restype = _i
@@ -70,7 +72,7 @@ _lib.ckopt_error_string.restype = ctypes.c_char_p
 _lib.ckopt_error_string.argtypes = [_i]
 
 EXPORTED_SYMBOLS = [
-    "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_1",
+    "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_2_lp", "ckopt_gemm_shmem_tc_async_opt_port_1",
     "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
     "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks", "ckopt_probe_counters",
@@ -157,6 +159,16 @@ def gemm_shmem_tc_async_opt_port(dtype, A, B, C, D, alpha, beta, M, N, K, tile_d
         dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
         bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
         num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port")
+
+
+def gemm_shmem_tc_async_opt_port_lp(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+                                    bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages,
+                                    num_producer_warps, num_consumer_warps, num_sms, stream=None):
+    """The <half, half> instance of the port_2 launcher (port_2.cu:968-1055): C and D in the operands' 16-bit type."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_2_lp(
+        dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+        bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+        num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port <DT, DT>")
 
 
 def gemm_shmem_tc_async_opt_port_1(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_step_rows_a,

@@ -68,13 +68,13 @@ __global__ void pad_rows_kernel(const unsigned short* __restrict__ src, unsigned
     }
 }
 
-int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta, int M,
-                int N, int K, const ck::GemmTuning& t, void* stream);
+int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
+                int N, int K, const ck::GemmTuning& t, void* stream, int out16);
 
 // K % 8 != 0 or operands off a 16-byte boundary: the product is computed from zero-padded,
 // aligned copies of A and Bt in a stream-ordered temporary (zeros in the K tail add nothing).
-int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta,
-                         int M, int N, int K, const ck::GemmTuning& t, void* stream) {
+int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta,
+                         int M, int N, int K, const ck::GemmTuning& t, void* stream, int out16) {
     using namespace ck;
     const int Kp = (K + CHUNK_ELEMS - 1) / CHUNK_ELEMS * CHUNK_ELEMS;
     const size_t bytes_a = (size_t)M * Kp * 2, bytes_b = (size_t)N * Kp * 2;
@@ -88,13 +88,13 @@ int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const float* 
     hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks((long long)M * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(A), pa, M, K, Kp);
     hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks((long long)N * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(Bt), pb, N, K, Kp);
     int rc = hipGetLastError() == hipSuccess ? CK_OK : CK_ERR_HIP;
-    if (rc == CK_OK) rc = gemm_launch(dtype, pa, pb, C, D, alpha, beta, M, N, Kp, t, stream);
+    if (rc == CK_OK) rc = gemm_launch(dtype, pa, pb, C, D, alpha, beta, M, N, Kp, t, stream, out16);
     if (hipFreeAsync(ws, s) != hipSuccess && rc == CK_OK) rc = CK_ERR_HIP;
     return rc;
 }
 
-int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta, int M,
-                int N, int K, const ck::GemmTuning& t, void* stream) {
+int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
+                int N, int K, const ck::GemmTuning& t, void* stream, int out16) {
     using namespace ck;
     if (!(dtype == CK_DT_F16 || dtype == CK_DT_BF16)) return CK_ERR_BAD_PARAM;
     if (M <= 0 || N <= 0 || K <= 0) return CK_ERR_BAD_PARAM;
@@ -103,16 +103,18 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float*
     if (!A || !Bt || !D) return CK_ERR_NULL;
     if (beta != 0.f && !C) return CK_ERR_NULL;
     if (((uintptr_t)A & 1) || ((uintptr_t)Bt & 1)) return CK_ERR_ALIGNMENT;
-    if (((uintptr_t)D & 3) || ((uintptr_t)C & 3)) return CK_ERR_ALIGNMENT;
+    const uintptr_t elem_mask = out16 ? 1 : 3;
+    if (((uintptr_t)D & elem_mask) || ((uintptr_t)C & elem_mask)) return CK_ERR_ALIGNMENT;
     // the kernels want every operand row on a 16-byte boundary
     if (K % CHUNK_ELEMS != 0 || ((uintptr_t)A & 15) || ((uintptr_t)Bt & 15))
-        return gemm_launch_repacked(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream);
+        return gemm_launch_repacked(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, out16);
     // one tile's rows are addressed through a 32-bit buffer offset
     if ((int64_t)t.tile_dim * K * 2 >= (int64_t)1 << 31) return CK_ERR_TOO_LARGE;
 
     const int mode = sync_mode_of(t.tile_dim, t.num_consumer_waves, t.bar_step_rows_a, t.bar_step_rows_b);
     GemmArgs a{};
-    a.A = A; a.Bt = Bt; a.C = C; a.D = D;
+    a.A = A; a.Bt = Bt; a.C = static_cast<const float*>(C); a.D = static_cast<float*>(D);
+    a.out16 = out16 ? 1 : 0;
     a.alpha = alpha; a.beta = beta;
     a.M = M; a.N = N; a.K = K;
     a.tiles_m = (M + t.tile_dim - 1) / t.tile_dim;
@@ -126,7 +128,8 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const float* C, float*
     a.bar_steps_b = mode == CK_SYNC_TILE ? 0 : t.bar_steps_b;
     a.swizzle = g_swizzle.load();
     a.num_xcd = g_num_xcd.load();
-    a.vec_store = (N % 4 == 0) && !((uintptr_t)D & 15) && (beta == 0.f || !((uintptr_t)C & 15));
+    const uintptr_t vec_mask = out16 ? 7 : 15;  // one 8- or 16-byte access per accumulator block
+    a.vec_store = (N % 4 == 0) && !((uintptr_t)D & vec_mask) && (beta == 0.f || !((uintptr_t)C & vec_mask));
     a.spin_limit = (uint32_t)g_spin_limit.load();
     a.prio_mode = g_prio_mode.load();
     a.producer_nap = g_producer_nap.load();
@@ -166,7 +169,17 @@ int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* B
                                          int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
     const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
                            tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream);
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0);
+}
+
+int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim,
+                                            int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                                            int bar_step_rows_b, int tile_group_m, int num_stages,
+                                            int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 1);
 }
 
 int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
@@ -185,7 +198,7 @@ int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* B
     }
     const ck::GemmTuning t{tile_dim, segment_dim_k, sa, sb, bar_step_rows_a, bar_step_rows_b,
                            tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream);
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0);
 }
 
 int ckopt_gemm_shmem_tc_async_opt_port_0(int dtype, const void* A, const void* Bt, const float* C, float* D,
@@ -194,7 +207,7 @@ int ckopt_gemm_shmem_tc_async_opt_port_0(int dtype, const void* A, const void* B
                                          int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
     const ck::GemmTuning t{tile_dim, segment_dim_k, 0, 0, tile_dim, tile_dim,
                            tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream);
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0);
 }
 
 int ckopt_get_lds_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,

@@ -230,32 +230,15 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
         const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
         const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
-        const float alpha = g.alpha, beta = g.beta;
         const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
 #pragma unroll
         for (int i = 0; i < WTR; ++i) {
-            const int m = m_base + i * 16;
 #pragma unroll
             for (int j = 0; j < WTC; ++j) {
-                const int n = n_base + j * 16;
-                const int64_t off = (int64_t)m * g.N + n;
-                f32x4 v = acc[i][j] * alpha;
 #if defined(CK_PROBE_NO_EPILOGUE)  // measurement build only: nothing is written (except by a workgroup that never exists)
-                if (blockIdx.x == 0x7fffffff) *(f32x4*)(g.D + off) = v;
+                if (blockIdx.x == 0x7fffffff) epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
 #else
-                if (interior) {
-                    if (beta != 0.f) v += *(const f32x4*)(g.C + off) * beta;
-                    *(f32x4*)(g.D + off) = v;
-                } else if (m < g.M) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (n + e < g.N) {
-                            float x = v[e];
-                            if (beta != 0.f) x += g.C[off + e] * beta;
-                            g.D[off + e] = x;
-                        }
-                    }
-                }
+                epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
 #endif
                 acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
             }

@@ -61,7 +61,8 @@ struct GemmArgs {
     int bar_steps_a, bar_steps_b;
     int swizzle;
     int num_xcd;
-    int vec_store;  // D (and C) 16-byte aligned with N % 4 == 0
+    int vec_store;  // D (and C) aligned for one vector access per accumulator block, N % 4 == 0
+    int out16;      // C and D hold the operands' 16-bit element type instead of fp32 (accumulation stays fp32)
     uint32_t spin_limit;
     int prio_mode;      // 0: producers at raised priority; 1: also asymmetric consumer burst priorities per SIMD pair; 2: none
     int producer_nap;   // s_sleep argument class of the producers' flag polling: 0 -> 1, 1 -> 4, 2 -> 16
@@ -84,6 +85,70 @@ template <> struct MfmaOp<bf16_tag> {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
 };
+
+// ---- epilogue of one 16 x 16 accumulator block: D = alpha * acc + beta * C. With the Bt fragment as the
+// first MFMA operand a lane holds 4 consecutive columns (n .. n+3) of one row m. C and D are fp32, or
+// (out16) the operands' 16-bit type: the sum is formed in fp32 and rounded to nearest even once.
+template <typename T> struct Out16;
+template <> struct Out16<f16_tag> {
+    static __device__ __forceinline__ float load(unsigned short b) { return (float)__builtin_bit_cast(_Float16, b); }
+    static __device__ __forceinline__ unsigned short store(float x) { return __builtin_bit_cast(unsigned short, (_Float16)x); }
+};
+template <> struct Out16<bf16_tag> {
+    static __device__ __forceinline__ float load(unsigned short b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+    static __device__ __forceinline__ unsigned short store(float x) {
+        uint32_t u = __builtin_bit_cast(uint32_t, x);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);  // NaN stays NaN
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (unsigned short)(u >> 16);
+    }
+};
+template <typename DT>
+__device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, f32x4 acc, bool interior) {
+    const int64_t off = (int64_t)m * g.N + n;
+    const float alpha = g.alpha, beta = g.beta;
+    f32x4 v = acc * alpha;
+    if (!g.out16) {
+        if (interior) {
+            if (beta != 0.f) v += *(const f32x4*)(g.C + off) * beta;
+            *(f32x4*)(g.D + off) = v;
+        } else if (m < g.M) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (n + e < g.N) {
+                    float x = v[e];
+                    if (beta != 0.f) x += g.C[off + e] * beta;
+                    g.D[off + e] = x;
+                }
+            }
+        }
+    } else {
+        const unsigned short* c16 = (const unsigned short*)g.C;
+        unsigned short* d16 = (unsigned short*)g.D;
+        if (interior) {
+            if (beta != 0.f) {
+                const uint2 c = *(const uint2*)(c16 + off);
+                v[0] += Out16<DT>::load((unsigned short)(c.x & 0xffffu)) * beta;
+                v[1] += Out16<DT>::load((unsigned short)(c.x >> 16)) * beta;
+                v[2] += Out16<DT>::load((unsigned short)(c.y & 0xffffu)) * beta;
+                v[3] += Out16<DT>::load((unsigned short)(c.y >> 16)) * beta;
+            }
+            uint2 o;
+            o.x = (uint32_t)Out16<DT>::store(v[0]) | ((uint32_t)Out16<DT>::store(v[1]) << 16);
+            o.y = (uint32_t)Out16<DT>::store(v[2]) | ((uint32_t)Out16<DT>::store(v[3]) << 16);
+            *(uint2*)(d16 + off) = o;
+        } else if (m < g.M) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (n + e < g.N) {
+                    float x = v[e];
+                    if (beta != 0.f) x += Out16<DT>::load(c16[off + e]) * beta;
+                    d16[off + e] = Out16<DT>::store(x);
+                }
+            }
+        }
+    }
+}
 
 // ---- LDS flag primitives (inline asm so the compiler's wait-count pass does not tie them to the
 // outstanding direct-to-LDS loads and force vmcnt(0) before every flag access) -------------------
@@ -606,30 +671,11 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
         // fragment as the first MFMA operand a lane holds 4 consecutive columns of one row.
         const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
         const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
-        const float alpha = g.alpha, beta = g.beta;
         const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
 #pragma unroll
         for (int i = 0; i < WTR; ++i) {
-            const int m = m_base + i * 16;
 #pragma unroll
-            for (int j = 0; j < WTC; ++j) {
-                const int n = n_base + j * 16;
-                const int64_t off = (int64_t)m * g.N + n;
-                f32x4 v = acc[i][j] * alpha;
-                if (interior) {
-                    if (beta != 0.f) v += *(const f32x4*)(g.C + off) * beta;
-                    *(f32x4*)(g.D + off) = v;
-                } else if (m < g.M) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (n + e < g.N) {
-                            float x = v[e];
-                            if (beta != 0.f) x += g.C[off + e] * beta;
-                            g.D[off + e] = x;
-                        }
-                    }
-                }
-            }
+            for (int j = 0; j < WTC; ++j) epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
         }
     }
 }

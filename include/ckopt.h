@@ -55,6 +55,16 @@ int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* B
                                          int bar_step_rows_b, int tile_group_m, int num_stages,
                                          int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
 
+/* The <half, half> role of the same launcher (the reference instantiates DT_ACC = half next to float,
+ * matmul_shmem_tc_async_opt_port_2.cu:968-1055): C and D hold the operands' 16-bit element type (fp16 for
+ * CKOPT_DT_F16, bf16 for CKOPT_DT_BF16; 2-byte aligned). Accumulation stays fp32; alpha * A * Bt^T + beta * C
+ * is rounded to nearest even once, so the result is at least as accurate as a 16-bit accumulator's. */
+int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim,
+                                            int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                                            int bar_step_rows_b, int tile_group_m, int num_stages,
+                                            int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
+
 /* Replaces gemm_shmem_tc_async_opt_port<DT,DT_ACC>() of matmul_shmem_tc_async_opt_port_1.cu:889-965:
  * every wave tile (or every 16-row block) has its own signal, i.e. port_2 with maximal bar_steps. */
 int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,

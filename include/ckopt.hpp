@@ -29,6 +29,16 @@ struct Error : std::runtime_error {
 };
 inline void check(int rc, const char* where) { if (rc != CKOPT_OK) throw Error(rc, where); }
 
+inline float to_float(float x) { return x; }
+inline float to_float(half_t x) { return (float)x; }
+inline float to_float(bfloat16_t x) {
+    const std::uint32_t u = (std::uint32_t)x.bits << 16;
+    float f;
+    static_assert(sizeof f == sizeof u, "");
+    __builtin_memcpy(&f, &u, sizeof f);
+    return f;
+}
+
 template <typename DT> struct dtype_of;
 template <> struct dtype_of<half_t> { static constexpr int value = CKOPT_DT_F16; };
 template <> struct dtype_of<bfloat16_t> { static constexpr int value = CKOPT_DT_BF16; };
@@ -41,11 +51,19 @@ void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B /* transposed: N x K 
                                   DT_ACC beta, int M, int N, int K, int tile_dim, int segment_dim_k, int bar_steps_a,
                                   int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
                                   int num_producer_warps, int num_consumer_warps, int num_sms, void* stream = nullptr) {
-    static_assert(std::is_same<DT_ACC, float>::value, "fp32 accumulate/output");
-    check(ckopt_gemm_shmem_tc_async_opt_port_2(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
-                                               bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m,
-                                               num_stages, num_producer_warps, num_consumer_warps, num_sms, stream),
-          "gemm_shmem_tc_async_opt_port");
+    static_assert(std::is_same<DT_ACC, float>::value || std::is_same<DT_ACC, DT>::value, "C / D are fp32 or the operand type");
+    if constexpr (std::is_same<DT_ACC, float>::value) {
+        check(ckopt_gemm_shmem_tc_async_opt_port_2(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
+                                                   bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m,
+                                                   num_stages, num_producer_warps, num_consumer_warps, num_sms, stream),
+              "gemm_shmem_tc_async_opt_port");
+    } else {  // the <half, half> instance: 16-bit C and D, alpha / beta given in that type
+        check(ckopt_gemm_shmem_tc_async_opt_port_2_lp(dtype_of<DT>::value, A, B, C, D, to_float(alpha), to_float(beta), M, N, K,
+                                                      tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
+                                                      bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+                                                      num_consumer_warps, num_sms, stream),
+              "gemm_shmem_tc_async_opt_port <DT, DT>");
+    }
 }
 // port_1: granularity only
 template <typename DT, typename DT_ACC>

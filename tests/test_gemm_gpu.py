@@ -401,3 +401,45 @@ def test_cpp_driver_through_the_launcher_templates(ck):
     assert "PASSED" in r.stdout and "correctness:" in r.stdout and "accuracy:" in r.stdout
     lines = [l for l in r.stdout.splitlines() if l.startswith("(") and "): " in l]
     assert len(lines) >= 8 and all(float(l.split("): ")[1]) > 1.0 for l in lines)
+
+
+# ---- the <half, half> role: C and D in the operands' 16-bit type, fp32 accumulation, one rounding ----------
+@pytest.mark.parametrize("dt_name", ["f16", "bf16"])
+def test_low_precision_output_instance(ck, oracle, dt_name):
+    dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16
+    odt = oracle.DT_F16 if dt_name == "f16" else oracle.DT_BF16
+    is_bf = dt_name == "bf16"
+    tdt = torch.bfloat16 if is_bf else torch.float16
+
+    def run(a, bt, c16, alpha, beta, t, M, N, K):
+        da, db = G.to_dev(a), G.to_dev(bt)
+        dc = None if c16 is None else G.to_dev(c16)
+        dd = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+        ck.gemm_shmem_tc_async_opt_port_lp(dt, da, db, dc, dd, alpha, beta, M, N, K, t["tile_dim"], t["segment_dim_k"],
+                                           t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                           t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                           t["num_consumer_warps"], t["num_sms"])
+        assert ck.device_status() == 0
+        return dd.float().cpu().numpy()
+
+    # exact: small integers, every value representable in 16 bits (|sum| <= 4 * 48 = 192 < 256)
+    M, N, K = 200, 264, 48
+    a = ck.fill_int(dt, (M, K), 71, 0, -2, 2)
+    bt = ck.fill_int(dt, (N, K), 71, 1, -2, 2)
+    want = (G.as_f64(is_bf, a) @ G.as_f64(is_bf, bt).T).astype(np.float32)
+    for t in (make_tuning(ck, 128, 32, 2, 2, 4), make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 64, 32, 3, 2, 8, "wave", 1, 1)):
+        assert np.array_equal(run(a, bt, None, 1.0, 0.0, t, M, N, K), want), t
+    # random, alpha / beta with a 16-bit C: fp32 result of the oracle, rounded once
+    M, N, K = 384, 512, 1024
+    a = ck.fill_uniform(dt, (M, K), 72, 0)
+    bt = ck.fill_uniform(dt, (N, K), 72, 1)
+    c16 = ck.fill_uniform(dt, (M, N), 72, 2)
+    cf = (G.bf16_bits_to_f32(c16) if is_bf else c16.astype(np.float32))
+    ref = oracle.gemm(odt, a, bt, cf, 0.75, -1.25)
+    ref16 = torch.from_numpy(ref).to(tdt).float().numpy()
+    for t in (make_tuning(ck, 256, 64, 2, 2, 8), make_tuning(ck, 128, 64, 3, 0, 4)):
+        got = run(a, bt, c16, 0.75, -1.25, t, M, N, K)
+        assert_close(oracle, ref, got)
+        # one rounding of an fp32 sum that differs from the oracle's only in summation order: at most 1 ulp apart
+        ulp = np.abs(ref16) * (2.0 ** -7 if is_bf else 2.0 ** -10) + 1e-3
+        assert np.all(np.abs(got - ref16) <= ulp)
