@@ -15,6 +15,8 @@ namespace ck {
 CK_DECL_GEMM(launch_gemm_pc_f16_m0) CK_DECL_GEMM(launch_gemm_pc_f16_m1) CK_DECL_GEMM(launch_gemm_pc_f16_m2)
 CK_DECL_GEMM(launch_gemm_pc_bf16_m0) CK_DECL_GEMM(launch_gemm_pc_bf16_m1) CK_DECL_GEMM(launch_gemm_pc_bf16_m2)
 #undef CK_DECL_GEMM
+hipError_t launch_gemm_pcb_f16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
+hipError_t launch_gemm_pcb_bf16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_fused_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_fused_bf16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_matmul_shmem(int dtype, int tile, int accs, bool bt, dim3 grid, hipStream_t s, const SimtArgs& a);
@@ -30,6 +32,7 @@ std::atomic<int> g_spin_limit{1 << 22};
 std::atomic<int> g_num_xcd{8};
 std::atomic<int> g_prio_mode{0};
 std::atomic<int> g_producer_nap{0};
+std::atomic<int> g_tile_sync_barrier{0};
 
 constexpr int MAX_DEV = 64;
 std::mutex g_status_mutex;
@@ -145,6 +148,11 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     if (t.num_producer_waves == 0) {
         e = dtype == CK_DT_F16 ? launch_gemm_fused_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a)
                                : launch_gemm_fused_bf16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a);
+    } else if (mode == CK_SYNC_TILE && t.num_stages >= 2 && g_tile_sync_barrier.load()) {
+        // tile granularity through the workgroup barrier: the ring is the whole LDS allocation
+        const size_t ring = (size_t)t.num_stages * 2 * stage_bytes_one_operand(t.tile_dim, t.segment_dim_k);
+        e = dtype == CK_DT_F16 ? launch_gemm_pcb_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, ring, s, a)
+                               : launch_gemm_pcb_bf16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, ring, s, a);
     } else if (dtype == CK_DT_F16) {
         if (mode == 0) e = launch_gemm_pc_f16_m0(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
         if (mode == 1) e = launch_gemm_pc_f16_m1(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, lds, s, a);
@@ -323,6 +331,7 @@ int ckopt_set_option(int key, int value) {
         case 2: if (value < 1 || value > 64) return ck::CK_ERR_BAD_PARAM; return g_num_xcd.exchange(value);
         case 3: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_prio_mode.exchange(value);
         case 4: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_producer_nap.exchange(value);
+        case 5: return g_tile_sync_barrier.exchange(value != 0);
         default: return ck::CK_ERR_BAD_PARAM;
     }
 }

@@ -142,7 +142,11 @@ int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, do
 
 /* Process-wide tuning switches that are not launcher parameters in the reference:
  * key 0: LDS XOR swizzle on/off (default 1); key 1: spin limit of bounded waits (default 1<<22);
- * key 2: number of XCDs assumed by the workgroup->tile remap (default 8; 1 disables the remap).
+ * key 2: number of XCDs assumed by the workgroup->tile remap (default 8; 1 disables the remap);
+ * key 3: wave priorities of the counter-synchronised kernel (0 producers raised (default), 1 also asymmetric
+ *        consumer bursts per SIMD pair, 2 none); key 4: producers' polling nap (0, 1, 2 = s_sleep 1, 4, 16);
+ * key 5: tile granularity with dedicated producers synchronises through the hardware workgroup barrier
+ *        (gemm_pcb_kernel, needs num_stages >= 2) instead of LDS counters (default 0).
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

@@ -443,3 +443,33 @@ def test_low_precision_output_instance(ck, oracle, dt_name):
         # one rounding of an fp32 sum that differs from the oracle's only in summation order: at most 1 ulp apart
         ulp = np.abs(ref16) * (2.0 ** -7 if is_bf else 2.0 ** -10) + 1e-3
         assert np.all(np.abs(got - ref16) <= ulp)
+
+
+@pytest.mark.parametrize("tile,c", [(64, 4), (64, 8), (128, 4), (128, 8), (256, 8)])
+def test_tile_sync_through_the_workgroup_barrier(ck, oracle, tile, c):
+    # option 5: dedicated producers, one hardware barrier per segment instead of LDS counters
+    prev = ck.set_option(ck.OPT_TILE_SYNC_BARRIER, 1)
+    try:
+        a = ck.fill_int(ck.DT_F16, (2 * tile, 640), 81, 0, -2, 2)
+        bt = ck.fill_int(ck.DT_F16, (3 * tile, 640), 81, 1, -2, 2)
+        want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)
+        ar = ck.fill_int(ck.DT_F16, (tile + 40, 72), 81, 2, -2, 2)
+        br = ck.fill_int(ck.DT_F16, (tile - 24, 72), 81, 3, -2, 2)
+        wantr = (ar.astype(np.int64) @ br.astype(np.int64).T).astype(np.float32)
+        n = 0
+        for sk, stages, p in itertools.product((32, 64, 128), (2, 3, 4), (2, 4, 8)):
+            t = make_tuning(ck, tile, sk, stages, p, c)
+            if not legal(ck, t):
+                continue
+            assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want), t
+            assert np.array_equal(G.run_gemm(ck, ck.DT_F16, ar, br, t=t), wantr), t
+            n += 1
+        assert n >= 4
+        M, N, K = 2 * tile, 2 * tile, 1024
+        a2 = ck.fill_uniform(ck.DT_BF16, (M, K), 82, 0)
+        b2 = ck.fill_uniform(ck.DT_BF16, (N, K), 82, 1)
+        c2 = ck.fill_uniform(ck.DT_F32, (M, N), 82, 2)
+        ref = oracle.gemm(oracle.DT_BF16, a2, b2, c2, 1.5, -0.5)
+        assert_close(oracle, ref, G.run_gemm(ck, ck.DT_BF16, a2, b2, c2, 1.5, -0.5, t=make_tuning(ck, tile, 32, 4, 4 if tile > 64 else 2, c)))
+    finally:
+        ck.set_option(ck.OPT_TILE_SYNC_BARRIER, prev)
