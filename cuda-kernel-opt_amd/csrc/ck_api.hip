@@ -17,6 +17,9 @@ CK_DECL_GEMM(launch_gemm_pc_bf16_m0) CK_DECL_GEMM(launch_gemm_pc_bf16_m1) CK_DEC
 #undef CK_DECL_GEMM
 hipError_t launch_gemm_pcb_f16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_pcb_bf16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
+hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a);
+hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a);
+bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves);
 hipError_t launch_gemm_fused_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_fused_bf16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_matmul_shmem(int dtype, int tile, int accs, bool bt, dim3 grid, hipStream_t s, const SimtArgs& a);
@@ -33,6 +36,7 @@ std::atomic<int> g_num_xcd{8};
 std::atomic<int> g_prio_mode{0};
 std::atomic<int> g_producer_nap{0};
 std::atomic<int> g_tile_sync_barrier{0};
+std::atomic<int> g_straight_line{1};
 
 constexpr int MAX_DEV = 64;
 std::mutex g_status_mutex;
@@ -145,7 +149,10 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     const size_t lds = (size_t)gemm_lds_bytes(t);
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
-    if (t.num_producer_waves == 0) {
+    if (g_straight_line.load() &&
+        gemm_stream_applies(a, t.tile_dim, t.segment_dim_k, t.num_stages, t.num_producer_waves, t.num_consumer_waves)) {
+        e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a) : launch_gemm_stream_bf16(dim3(grid), s, a);
+    } else if (t.num_producer_waves == 0) {
         e = dtype == CK_DT_F16 ? launch_gemm_fused_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a)
                                : launch_gemm_fused_bf16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a);
     } else if (mode == CK_SYNC_TILE && t.num_stages >= 2 && g_tile_sync_barrier.load()) {
@@ -332,6 +339,7 @@ int ckopt_set_option(int key, int value) {
         case 3: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_prio_mode.exchange(value);
         case 4: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_producer_nap.exchange(value);
         case 5: return g_tile_sync_barrier.exchange(value != 0);
+        case 6: return g_straight_line.exchange(value != 0);
         default: return ck::CK_ERR_BAD_PARAM;
     }
 }

@@ -111,7 +111,11 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
     if (!g.out16) {
         if (interior) {
             if (beta != 0.f) v += *(const f32x4*)(g.C + off) * beta;
+#if defined(CK_NT_STORE)  // D is written once and not read again: keep it from displacing the operands in L2
+            __builtin_nontemporal_store(v, (f32x4*)(g.D + off));
+#else
             *(f32x4*)(g.D + off) = v;
+#endif
         } else if (m < g.M) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -136,7 +140,12 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
             uint2 o;
             o.x = (uint32_t)Out16<DT>::store(v[0]) | ((uint32_t)Out16<DT>::store(v[1]) << 16);
             o.y = (uint32_t)Out16<DT>::store(v[2]) | ((uint32_t)Out16<DT>::store(v[3]) << 16);
+#if defined(CK_NT_STORE)
+            __builtin_nontemporal_store(o.x, (uint32_t*)(d16 + off));
+            __builtin_nontemporal_store(o.y, (uint32_t*)(d16 + off) + 1);
+#else
             *(uint2*)(d16 + off) = o;
+#endif
         } else if (m < g.M) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {

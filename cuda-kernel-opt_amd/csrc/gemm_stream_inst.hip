@@ -1,0 +1,33 @@
+// Launchers of the straight-line 256 x 256 kernel (one instance per element type).
+#define CK_NT_STORE 1
+#include "gemm_stream_kernel.hip.h"
+
+namespace ck {
+
+template <typename DT>
+static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a) {
+    auto kern = gemm_stream_kernel<DT>;
+    static bool opted[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64 && !opted[dev]) {
+        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES_PER_CU);
+        if (e != hipSuccess) return e;
+        opted[dev] = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(512), STREAM_LDS_BYTES, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a) { return stream_launch<f16_tag>(grid, stream, a); }
+hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a) { return stream_launch<bf16_tag>(grid, stream, a); }
+
+// what the kernel assumes about a launch (the caller falls back to the general fused kernel otherwise)
+bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves) {
+    return producer_waves == 0 && consumer_waves == 8 && tile_dim == STREAM_TILE && segment_dim_k == STREAM_SEGK &&
+           num_stages == STREAM_STAGES && a.M % STREAM_TILE == 0 && a.N % STREAM_TILE == 0 && a.K % STREAM_K_MULTIPLE == 0 &&
+           a.vec_store && a.swizzle;
+}
+
+}  // namespace ck

@@ -1,0 +1,286 @@
+// The straight-line form of the fused (no dedicated producer waves) kernel for the shape the headline
+// sizes use: 256 x 256 tiles, eight waves, whole tiles only (M and N multiples of 256), K a multiple
+// of 64, and a ring of five 32-deep K segments ("quarters", 32 KiB each) - all of the CU's LDS. With
+// those fixed the loop body is two k-steps, the loader runs exactly two bodies ahead of the
+// multiplier, and every wait is an immediate - no mode flags, no wait ladder, no per-segment
+// bookkeeping between the MFMAs.
+//
+// Why five quarters and "pair fetch": a 32-deep segment is 64 bytes of each operand row, half a
+// cache line. Fetching the halves in different k-steps makes the L1 ask the L2 for every line twice
+// (measured: 17.9 TB/s of useful bytes for this access pattern against 26 TB/s with whole lines -
+// below what the MFMAs consume at full rate). So a wave fetches both halves of its rows back to back
+// (the second request merges with the first in the L1) into two quarters at once, every second
+// k-step. Four quarters would leave two k-steps between issue and use, as a ring of two 64-deep
+// stages does; the fifth buys a third.
+//
+// Even k-step j (quarter q = j % 5), fragments of j on their way to registers:
+//     fragments in registers; first column of MFMAs; workgroup barrier -> quarter q is free
+//     7 columns of MFMAs; under them the fragments of j+1 from quarter q+1 and this wave's eight
+//     loads of k-steps j+4 and j+5 into quarters q+4 (free since the previous barrier) and q
+// Odd k-step j+1:
+//     fragments in registers; own loads of k-steps j+2, j+3 landed (the eight just issued may fly);
+//     first column; barrier -> quarters q+2, q+3 complete; 7 columns, fragments of j+2 from q+2
+// The stream of k-steps runs across the tiles of the persistent workgroup; the loader moves to the
+// next tile two bodies before the multiplier does, so its first quarters are in flight while the
+// current tile is finished and written out.
+//
+// Vector memory operations of a wave complete in issue order, stores included, so "the loads of
+// k-step X have landed" is "at most as many operations outstanding as were issued after them".
+// In the body that follows an epilogue the 32 stores of the epilogue sit between the loads already
+// in flight and the new ones, and the immediate accounts for them - waiting for the stores
+// themselves would put their whole latency in front of the first MFMAs of every tile.
+#ifndef CK_GEMM_STREAM_KERNEL_HIP_H
+#define CK_GEMM_STREAM_KERNEL_HIP_H
+
+#include "gemm_fused_kernel.hip.h"
+
+namespace ck {
+
+constexpr int STREAM_TILE = 256;
+constexpr int STREAM_SEGK = 32;
+constexpr int STREAM_STAGES = 5;
+constexpr int STREAM_K_MULTIPLE = 2 * STREAM_SEGK;  // one loop body
+constexpr int STREAM_LDS_BYTES = STREAM_STAGES * 2 * STREAM_TILE * STREAM_SEGK * 2;
+
+template <typename DT>
+__global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
+    constexpr int TILE = STREAM_TILE, NQ = STREAM_STAGES;
+    constexpr int WTR = 4, WTC = 8;          // 16 x 16 blocks per wave tile (64 x 128)
+    constexpr int RB = STREAM_SEGK * 2;      // bytes per LDS row
+    constexpr int OPB = TILE * RB;           // one operand's part of a quarter
+    constexpr int QB = 2 * OPB;              // one quarter
+    constexpr int LPB = 8;                   // loads per wave and body: (A, Bt) x (rows w, w + 8) x (two halves)
+    constexpr int EPILOGUE_STORES = WTR * WTC;
+    static_assert(LPB + EPILOGUE_STORES < 64, "the wait immediates must fit the 6-bit counter");
+    static_assert(STREAM_LDS_BYTES <= LDS_BYTES_PER_CU, "the ring is all of the LDS");
+
+    extern __shared__ __attribute__((aligned(1024))) char ck_smem[];
+    const uint32_t ring_base = (uint32_t)(uintptr_t)(CK_LDS char*)ck_smem;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const unsigned long long clk0 = clock64(), wall0 = wall_clock64();
+
+    const int grid = gridDim.x;
+    const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
+    const int total_tiles = g.tiles_m * g.tiles_n;
+    const int my_tiles = slot < total_tiles ? (total_tiles - slot + grid - 1) / grid : 0;
+    const int nb = g.K / STREAM_K_MULTIPLE;  // loop bodies per tile
+
+    // ---- loader ------------------------------------------------------------------------------------
+    // A wave load covers 16 rows x 64 bytes of an operand quarter; wave w issues the loads of rows
+    // 16w.. and 16(w+8).. of A and of Bt. Lane (row, slot) fetches the 16-byte chunk that belongs at
+    // its linear LDS position under the XOR swizzle (the key depends on the row inside the 16-row
+    // block only).
+    const uint32_t pitch32 = (uint32_t)g.K * 2u;
+    const int lane_row = lane / 4, lane_slot = lane % 4;
+    const uint32_t loff = (uint32_t)lane_row * pitch32 + (uint32_t)swizzle_slot(lane_row, lane_slot, 4, 1) * CHUNK_BYTES;
+    const uint32_t dst_w = ring_base + (uint32_t)wave * 1024u;
+    const uint32_t goff_w = (uint32_t)wave * 16u * pitch32;
+    const uint32_t goff_hi = 8u * 16u * pitch32;   // rows 16(w+8).. relative to rows 16w..
+    const uint32_t nrec = (uint32_t)TILE * pitch32;
+    i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // empty descriptors: loads read zeros
+    uint32_t l_koff = 0;  // byte offset along K of the body being loaded
+    int l_tile = 0;       // index (in this workgroup's list) of the tile being loaded
+    auto loader_open_tile = [&]() __attribute__((always_inline)) {
+        if (l_tile < my_tiles) {
+            const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, slot + (int64_t)l_tile * grid);
+            const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE);
+            rsrc_a = make_rsrc((const char*)g.A + (int64_t)row_a * pitch32, nrec);
+            rsrc_b = make_rsrc((const char*)g.Bt + (int64_t)row_b * pitch32, nrec);
+        } else {
+            rsrc_a[2] = 0;  // past the last tile: nothing is fetched (the ring receives zeros nobody reads)
+            rsrc_b[2] = 0;
+        }
+    };
+    auto loader_advance = [&]() __attribute__((always_inline)) {
+        l_koff += STREAM_K_MULTIPLE * 2;
+        if (l_koff == pitch32) {
+            l_koff = 0;
+            ++l_tile;
+            loader_open_tile();
+        }
+    };
+    // Load pair P (0, 1: A rows 16w.. / 16(w+8)..; 2, 3: Bt likewise) of the body at l_koff: the two
+    // halves of each row's line, back to back, into the quarters at byte offsets q_lo and q_hi.
+    auto issue_pair = [&](auto index, uint32_t q_lo, uint32_t q_hi) __attribute__((always_inline)) {
+        constexpr int P = decltype(index)::value;
+        constexpr bool IS_A = P < 2;
+        constexpr int HI = P % 2;
+        const uint32_t dst = dst_w + (uint32_t)((IS_A ? 0 : OPB) + HI * 8 * 1024);
+        const uint32_t soff = goff_w + (HI ? goff_hi : 0u) + l_koff;
+        dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_lo, loff, soff);
+        dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_hi, loff, soff + (uint32_t)(STREAM_SEGK * 2));
+    };
+
+    // ---- multiplier --------------------------------------------------------------------------------
+    const int R = wave / 2, Cc = wave % 2;
+    const int lr = lane & 15, lg = lane >> 4;
+    const int key = swizzle_key(lr, 4);
+    const uint32_t a_lane = ring_base + (uint32_t)(R * WTR * 16 + lr) * RB + (uint32_t)((lg ^ key) * CHUNK_BYTES);
+    const uint32_t b_lane = ring_base + (uint32_t)OPB + (uint32_t)(Cc * WTC * 16 + lr) * RB + (uint32_t)((lg ^ key) * CHUNK_BYTES);
+
+    u32x4 fa[2][WTR], fb[2][WTC];
+    f32x4 acc[WTR][WTC];
+#pragma unroll
+    for (int i = 0; i < WTR; ++i)
+#pragma unroll
+        for (int j = 0; j < WTC; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // 1 when beta is (plus or minus) zero: then the epilogue is 32 stores and nothing else. Worked out on
+    // the scalar unit in asm: a flag the compiler derives from a float compare ends up in a vector
+    // register, which the "s" operands of the asm statements below cannot take.
+    uint32_t count_stores;
+    asm volatile("s_lshl_b32 %0, %1, 1\n\ts_cmp_eq_u32 %0, 0\n\ts_cselect_b32 %0, 1, 0"
+                 : "=&s"(count_stores)
+                 : "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, g.beta)))
+                 : "scc");
+#if defined(CK_PROBE_TIMING)  // measurement build only: cycles in the epilogues, in the first and second loop body behind one, in all others
+    unsigned long long t_epi = 0, t_first = 0, t_second = 0, t_other = 0;
+#endif
+    uint32_t stores_in_flight;  // nonzero in the loop body that follows an epilogue whose stores count in the wait
+    asm volatile("s_mov_b32 %0, 0" : "=s"(stores_in_flight));
+    // byte offsets in the ring of the quarters of the even k-step (q0) and of the four after it
+    uint32_t q0 = 0, q1 = QB, q2 = 2 * QB, q4 = 4 * QB;
+
+    // One k-step: P selects the fragment buffers; qn is the quarter of the next k-step (its fragments
+    // are fetched here); the even k-step also issues the body's loads into quarters q4 and q0.
+    auto kstep = [&](auto parity, uint32_t qn) __attribute__((always_inline)) {
+        constexpr int P = decltype(parity)::value;
+        use_fragments(fa[P], fb[P]);
+#if !defined(CK_PROBE_NO_LANDING_WAIT)  // measurement builds drop the wait (results are wrong)
+        if constexpr (P == 1) {
+            // loads of the next two k-steps landed: after them this wave issued this body's eight
+            // loads and, behind an epilogue, the epilogue's stores. (The choice between the two
+            // immediates is a scalar branch inside one asm statement: a branch the compiler can see
+            // would split the k-step into basic blocks with all 224 accumulator and fragment
+            // registers live across them.)
+            asm volatile("s_cmp_lg_u32 %0, 0\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(%1)\n1:\n\ts_waitcnt vmcnt(%2)"
+                         :
+                         : "s"(stores_in_flight), "n"(LPB), "n"(LPB + EPILOGUE_STORES)
+                         : "memory", "scc");
+        }
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < WTR; ++i) acc[i][0] = MfmaOp<DT>::run(fb[P][0], fa[P][i], acc[i][0]);
+        __builtin_amdgcn_sched_barrier(0);
+        wg_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t pa = a_lane + qn, pb = b_lane + qn;
+#pragma unroll
+        for (int j = 1; j < WTC; ++j) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int f = (j - 1) * 2 + q;
+                if (f < WTR) fa[1 - P][f] = *(const CK_LDS u32x4*)(uintptr_t)(pa + (uint32_t)(f * 16 * RB));
+                else if (f < WTR + WTC) fb[1 - P][f - WTR] = *(const CK_LDS u32x4*)(uintptr_t)(pb + (uint32_t)((f - WTR) * 16 * RB));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (P == 0) {
+                if (j == 1) issue_pair(std::integral_constant<int, 0>{}, q4, q0);
+                if (j == 3) issue_pair(std::integral_constant<int, 1>{}, q4, q0);
+                if (j == 5) issue_pair(std::integral_constant<int, 2>{}, q4, q0);
+                if (j == 7) issue_pair(std::integral_constant<int, 3>{}, q4, q0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+#if defined(CK_STAGGER_CLASSES)  // tuning builds: workgroups start in classes, CK_STAGGER_STEP_US apart
+    {
+#if defined(CK_STAGGER_BY_XCD)
+        const int cls = (int)(blockIdx.x % 8) % CK_STAGGER_CLASSES;
+#else
+        const int cls = (int)(blockIdx.x / 8) % CK_STAGGER_CLASSES;
+#endif
+        const unsigned long long until = wall0 + (unsigned long long)cls * (CK_STAGGER_STEP_US * 100);
+        while (wall_clock64() < until) __builtin_amdgcn_s_sleep(8);
+    }
+#endif
+    if (my_tiles > 0) {
+        // prologue: the first two bodies' quarters, then the fragments of k-step 0
+        loader_open_tile();
+        issue_pair(std::integral_constant<int, 0>{}, 0u, (uint32_t)QB);
+        issue_pair(std::integral_constant<int, 1>{}, 0u, (uint32_t)QB);
+        issue_pair(std::integral_constant<int, 2>{}, 0u, (uint32_t)QB);
+        issue_pair(std::integral_constant<int, 3>{}, 0u, (uint32_t)QB);
+        loader_advance();
+        issue_pair(std::integral_constant<int, 0>{}, (uint32_t)(2 * QB), (uint32_t)(3 * QB));
+        issue_pair(std::integral_constant<int, 1>{}, (uint32_t)(2 * QB), (uint32_t)(3 * QB));
+        issue_pair(std::integral_constant<int, 2>{}, (uint32_t)(2 * QB), (uint32_t)(3 * QB));
+        issue_pair(std::integral_constant<int, 3>{}, (uint32_t)(2 * QB), (uint32_t)(3 * QB));
+        loader_advance();
+        wait_vmcnt_imm<LPB>();
+        wg_barrier();
+#pragma unroll
+        for (int i = 0; i < WTR; ++i) fa[0][i] = *(const CK_LDS u32x4*)(uintptr_t)(a_lane + (uint32_t)(i * 16 * RB));
+#pragma unroll
+        for (int j = 0; j < WTC; ++j) fb[0][j] = *(const CK_LDS u32x4*)(uintptr_t)(b_lane + (uint32_t)(j * 16 * RB));
+
+        for (int t = 0; t < my_tiles; ++t) {
+            for (int b = 0; b < nb; ++b) {
+#if defined(CK_PROBE_TIMING)
+                const unsigned long long tb0 = clock64();
+#endif
+                kstep(std::integral_constant<int, 0>{}, q1);
+                loader_advance();
+                kstep(std::integral_constant<int, 1>{}, q2);
+                asm volatile("s_mov_b32 %0, 0" : "=s"(stores_in_flight));
+                // two quarters on: q0 <- q2, q1 <- q3 = q4 - QB (mod ring), q2 <- q4, q4 <- q1
+                {
+                    const uint32_t n0 = q2, n2 = q4, n4 = q1;
+                    uint32_t n1 = q2 + QB;
+                    if (n1 == (uint32_t)(NQ * QB)) n1 = 0;
+                    q0 = n0; q1 = n1; q2 = n2; q4 = n4;
+                }
+#if defined(CK_PROBE_TIMING)
+                { const unsigned long long d = clock64() - tb0; if (b == 0 && t > 0) t_first += d; else if (b == 1 && t > 0) t_second += d; else t_other += d; }
+#endif
+            }
+#if defined(CK_PROBE_TIMING)
+            const unsigned long long te0 = clock64();
+#endif
+            // D = alpha * acc + beta * C straight from the accumulators
+            const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, slot + (int64_t)t * grid);
+            const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
+            const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
+#pragma unroll
+            for (int i = 0; i < WTR; ++i) {
+#pragma unroll
+                for (int j = 0; j < WTC; ++j) {
+#if defined(CK_PROBE_NO_EPILOGUE)  // measurement build only: nothing is written (except by a workgroup that never exists)
+                    if (blockIdx.x == 0x7fffffff)
+#endif
+                    epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], true);
+                    acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+#if defined(CK_PROBE_TIMING)
+            t_epi += clock64() - te0;
+#endif
+            // (set through asm so that the flag stays one opaque scalar register: otherwise the compiler
+            // peels the loop around its known values)
+            asm volatile("s_mov_b32 %0, %1" : "=s"(stores_in_flight) : "s"(count_stores));
+        }
+        // the loads issued past the last tile fetch nothing, but they still write the ring
+        wait_vmcnt_imm<0>();
+    }
+
+#if defined(CK_PROBE_TIMING)
+    if (blockIdx.x == 0 && lane == 0) {
+        unsigned* o = g.status + 8 + wave * 8;
+        o[0] = (unsigned)(t_epi >> 4); o[1] = (unsigned)(t_first >> 4); o[2] = (unsigned)(t_second >> 4); o[3] = (unsigned)(t_other >> 4);
+    }
+#endif
+    if (blockIdx.x == 0 && threadIdx.x == blockDim.x - 1) {
+        const unsigned long long dc = clock64() - clk0, dw = wall_clock64() - wall0;
+        g.status[2] = (unsigned)dc; g.status[3] = (unsigned)(dc >> 32);
+        g.status[4] = (unsigned)dw; g.status[5] = (unsigned)(dw >> 32);
+    }
+}
+
+}  // namespace ck
+#endif  // CK_GEMM_STREAM_KERNEL_HIP_H
