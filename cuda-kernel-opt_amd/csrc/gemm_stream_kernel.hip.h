@@ -15,11 +15,12 @@
 //
 // Even k-step j (quarter q = j % 5), fragments of j on their way to registers:
 //     fragments in registers; first column of MFMAs; workgroup barrier -> quarter q is free
-//     7 columns of MFMAs; under them the fragments of j+1 from quarter q+1 and this wave's eight
-//     loads of k-steps j+4 and j+5 into quarters q+4 (free since the previous barrier) and q
+//     7 columns of MFMAs; under them the fragments of j+1 from quarter q+1 and this wave's four
+//     loads of A for k-steps j+4 and j+5 into quarters q+4 (free since the previous barrier) and q
 // Odd k-step j+1:
-//     fragments in registers; own loads of k-steps j+2, j+3 landed (the eight just issued may fly);
-//     first column; barrier -> quarters q+2, q+3 complete; 7 columns, fragments of j+2 from q+2
+//     fragments in registers; own loads of k-steps j+2, j+3 landed (the four just issued may fly);
+//     first column; barrier -> quarters q+2, q+3 complete; 7 columns, fragments of j+2 from q+2 and
+//     the four loads of Bt for k-steps j+4 and j+5
 // The stream of k-steps runs across the tiles of the persistent workgroup; the loader moves to the
 // next tile two bodies before the multiplier does, so its first quarters are in flight while the
 // current tile is finished and written out.
@@ -83,7 +84,11 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     int l_tile = 0;       // index (in this workgroup's list) of the tile being loaded
     auto loader_open_tile = [&]() __attribute__((always_inline)) {
         if (l_tile < my_tiles) {
+#if defined(CK_PROBE_SAME_TILE)  // measurement build only: every workgroup loads the operands of tile (0, 0)
+            const TileRC rc{0, 0};
+#else
             const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, slot + (int64_t)l_tile * grid);
+#endif
             const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE);
             rsrc_a = make_rsrc((const char*)g.A + (int64_t)row_a * pitch32, nrec);
             rsrc_b = make_rsrc((const char*)g.Bt + (int64_t)row_b * pitch32, nrec);
@@ -143,20 +148,20 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     uint32_t q0 = 0, q1 = QB, q2 = 2 * QB, q4 = 4 * QB;
 
     // One k-step: P selects the fragment buffers; qn is the quarter of the next k-step (its fragments
-    // are fetched here); the even k-step also issues the body's loads into quarters q4 and q0.
+    // are fetched here); its loads go into quarters q4 and q0.
     auto kstep = [&](auto parity, uint32_t qn) __attribute__((always_inline)) {
         constexpr int P = decltype(parity)::value;
         use_fragments(fa[P], fb[P]);
 #if !defined(CK_PROBE_NO_LANDING_WAIT)  // measurement builds drop the wait (results are wrong)
         if constexpr (P == 1) {
-            // loads of the next two k-steps landed: after them this wave issued this body's eight
-            // loads and, behind an epilogue, the epilogue's stores. (The choice between the two
-            // immediates is a scalar branch inside one asm statement: a branch the compiler can see
-            // would split the k-step into basic blocks with all 224 accumulator and fragment
-            // registers live across them.)
+            // loads of the next two k-steps landed: after them this wave issued the four loads of
+            // this body's even k-step and, behind an epilogue, the epilogue's stores. (The choice
+            // between the two immediates is a scalar branch inside one asm statement: a branch the
+            // compiler can see would split the k-step into basic blocks with all 224 accumulator
+            // and fragment registers live across them.)
             asm volatile("s_cmp_lg_u32 %0, 0\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(%1)\n1:\n\ts_waitcnt vmcnt(%2)"
                          :
-                         : "s"(stores_in_flight), "n"(LPB), "n"(LPB + EPILOGUE_STORES)
+                         : "s"(stores_in_flight), "n"(LPB / 2), "n"(LPB / 2 + EPILOGUE_STORES)
                          : "memory", "scc");
         }
 #endif
@@ -176,12 +181,11 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                 else if (f < WTR + WTC) fb[1 - P][f - WTR] = *(const CK_LDS u32x4*)(uintptr_t)(pb + (uint32_t)((f - WTR) * 16 * RB));
             }
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (P == 0) {
-                if (j == 1) issue_pair(std::integral_constant<int, 0>{}, q4, q0);
-                if (j == 3) issue_pair(std::integral_constant<int, 1>{}, q4, q0);
-                if (j == 5) issue_pair(std::integral_constant<int, 2>{}, q4, q0);
-                if (j == 7) issue_pair(std::integral_constant<int, 3>{}, q4, q0);
-            }
+            // this k-step's share of the loads, one pair behind every third column: the pairs of A in the
+            // even k-step, those of Bt in the odd one (a wave stalls on back-to-back loads, and both waves
+            // of a SIMD run in step)
+            if (j == 3) issue_pair(std::integral_constant<int, 2 * P>{}, q4, q0);
+            if (j == 6) issue_pair(std::integral_constant<int, 2 * P + 1>{}, q4, q0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
@@ -189,17 +193,6 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         }
     };
 
-#if defined(CK_STAGGER_CLASSES)  // tuning builds: workgroups start in classes, CK_STAGGER_STEP_US apart
-    {
-#if defined(CK_STAGGER_BY_XCD)
-        const int cls = (int)(blockIdx.x % 8) % CK_STAGGER_CLASSES;
-#else
-        const int cls = (int)(blockIdx.x / 8) % CK_STAGGER_CLASSES;
-#endif
-        const unsigned long long until = wall0 + (unsigned long long)cls * (CK_STAGGER_STEP_US * 100);
-        while (wall_clock64() < until) __builtin_amdgcn_s_sleep(8);
-    }
-#endif
     if (my_tiles > 0) {
         // prologue: the first two bodies' quarters, then the fragments of k-step 0
         loader_open_tile();
@@ -226,8 +219,8 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                 const unsigned long long tb0 = clock64();
 #endif
                 kstep(std::integral_constant<int, 0>{}, q1);
-                loader_advance();
                 kstep(std::integral_constant<int, 1>{}, q2);
+                loader_advance();
                 asm volatile("s_mov_b32 %0, 0" : "=s"(stores_in_flight));
                 // two quarters on: q0 <- q2, q1 <- q3 = q4 - QB (mod ring), q2 <- q4, q4 <- q1
                 {

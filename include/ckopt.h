@@ -147,6 +147,9 @@ int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, do
  *        consumer bursts per SIMD pair, 2 none); key 4: producers' polling nap (0, 1, 2 = s_sleep 1, 4, 16);
  * key 5: tile granularity with dedicated producers synchronises through the hardware workgroup barrier
  *        (gemm_pcb_kernel, needs num_stages >= 2) instead of LDS counters (default 0).
+ * key 6: launches with num_producer_warps 0, tile_dim 256, segment_dim_k 32, num_stages 5, 8 consumer warps, whole
+ *        tiles (M, N multiples of 256) and K a multiple of 64 take the straight-line kernel written for exactly
+ *        that shape (gemm_stream_kernel; default 1); 0 sends them through the general fused kernel.
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

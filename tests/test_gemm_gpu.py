@@ -473,3 +473,71 @@ def test_tile_sync_through_the_workgroup_barrier(ck, oracle, tile, c):
         assert_close(oracle, ref, G.run_gemm(ck, ck.DT_BF16, a2, b2, c2, 1.5, -0.5, t=make_tuning(ck, tile, 32, 4, 4 if tile > 64 else 2, c)))
     finally:
         ck.set_option(ck.OPT_TILE_SYNC_BARRIER, prev)
+
+
+STRAIGHT_LINE = dict(tile=256, sk=32, stages=5, p=0, c=8)
+
+
+def _straight_line_tuning(ck, cus=256, group=4):
+    t = make_tuning(ck, STRAIGHT_LINE["tile"], STRAIGHT_LINE["sk"], STRAIGHT_LINE["stages"], STRAIGHT_LINE["p"], STRAIGHT_LINE["c"])
+    t["num_sms"] = cus
+    t["tile_group_m"] = group
+    return t
+
+
+@pytest.mark.parametrize("M,N,K,cus,group", [
+    (256, 256, 64, 256, 4),      # one tile, one loop body: prologue, one body, epilogue
+    (256, 256, 192, 256, 4),     # odd number of bodies: the ring position at a tile's end varies
+    (512, 768, 320, 256, 4),
+    (1024, 1024, 64, 3, 4),      # many tiles per workgroup, every body follows an epilogue
+    (1024, 1024, 192, 5, 4),
+    (1024, 1280, 1152, 7, 3),    # group size that does not divide the tile rows
+    (2048, 2048, 1024, 256, 4),
+])
+def test_straight_line_kernel_bit_exact(ck, M, N, K, cus, group):
+    t = _straight_line_tuning(ck, cus, group)
+    assert legal(ck, t)
+    for dt in (ck.DT_F16, ck.DT_BF16):
+        a = ck.fill_int(dt, (M, K), 91, 0, -2, 2)
+        bt = ck.fill_int(dt, (N, K), 91, 1, -2, 2)
+        want = (G.as_f64(dt == ck.DT_BF16, a) @ G.as_f64(dt == ck.DT_BF16, bt).T).astype(np.float32)
+        assert np.array_equal(G.run_gemm(ck, dt, a, bt, t=t), want)
+
+
+def test_straight_line_kernel_epilogue_and_general_kernel_agree(ck, oracle):
+    # beta != 0 (the epilogue reads C: the store accounting of the waits is off), 16-bit C/D, and the
+    # same launches through the general fused kernel (option 6 off) give the same bits
+    M, N, K = 768, 512, 448
+    t = _straight_line_tuning(ck, cus=2)
+    a = ck.fill_uniform(ck.DT_F16, (M, K), 92, 0)
+    bt = ck.fill_uniform(ck.DT_F16, (N, K), 92, 1)
+    c = ck.fill_uniform(ck.DT_F32, (M, N), 92, 2)
+    got = G.run_gemm(ck, ck.DT_F16, a, bt, c, 1.5, -0.5, t=t)
+    assert_close(oracle, oracle.gemm(oracle.DT_F16, a, bt, c, 1.5, -0.5), got)
+    ai = ck.fill_int(ck.DT_F16, (M, K), 93, 0, -2, 2)
+    bi = ck.fill_int(ck.DT_F16, (N, K), 93, 1, -2, 2)
+    ci = ck.fill_int(ck.DT_F32, (M, N), 93, 2, -3, 3)
+    want = 2.0 * (ai.astype(np.int64) @ bi.astype(np.int64).T) - ci.astype(np.float64)
+    assert np.array_equal(G.run_gemm(ck, ck.DT_F16, ai, bi, ci, 2.0, -1.0, t=t), want.astype(np.float32))
+    prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
+    try:
+        general = G.run_gemm(ck, ck.DT_F16, a, bt, c, 1.5, -0.5, t=t)
+    finally:
+        ck.set_option(ck.OPT_STRAIGHT_LINE, prev)
+    assert_close(oracle, general, got)
+
+
+def test_straight_line_kernel_headline_size_properties(ck):
+    # 8192^3 in the headline configuration: constant operands have a closed form (every output
+    # alpha * 10 * K), and a one-hot Bt picks columns of A exactly
+    M = N = K = 8192
+    t = _straight_line_tuning(ck)
+    a = ck.fill_constant(ck.DT_F16, (M, K), 1.0)
+    bt = ck.fill_constant(ck.DT_F16, (N, K), 10.0)
+    d = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+    assert float(d.min()) == float(d.max()) == 10.0 * K
+    a = ck.fill_int(ck.DT_F16, (M, K), 94, 0, -8, 8)
+    eye = np.zeros((N, K), dtype=np.float16)
+    eye[np.arange(N), (np.arange(N) * 5 + 3) % K] = 1.0
+    d = G.run_gemm(ck, ck.DT_F16, a, eye, t=t)
+    assert np.array_equal(d, a[:, (np.arange(N) * 5 + 3) % K].astype(np.float32))
