@@ -36,8 +36,8 @@ WORKLOADS = {
 TUNED = {
     "config1_fp16_512": (64, 128, 4, 0, 8),
     "config3_fp16_8192": (256, 32, 5, 0, 8),
-    "config4_fp16_2048x2048x32768": (128, 128, 2, 0, 8),
-    "config5_bf16_6143x4097x3071": (256, 64, 2, 2, 8),
+    "config4_fp16_2048x2048x32768": (256, 32, 5, 0, 8),
+    "config5_bf16_6143x4097x3071": (256, 32, 5, 0, 8),
     "config6_fp16_16384": (256, 32, 5, 0, 8),
 }
 
@@ -178,7 +178,7 @@ def main():
                                             args.producers, args.consumers, cus, stream)
         peak, bound_name, arith = PEAK_TFLOPS["mfma_f16"], "mfma", dtype
         if (args.producers == 0 and args.tile == 256 and args.segk == 32 and args.stages == 5 and args.consumers == 8
-                and M % 256 == 0 and N % 256 == 0 and K % 64 == 0):
+                and (K + 7) // 8 * 8 % 64 == 0):
             kernel = "gemm_stream_kernel<%s, tile 256, five 32-deep quarters, 8 waves, pair fetch>" % dtype
         elif args.producers == 0:
             kernel = "gemm_fused_kernel<%s, tile %d, seg_k %d, %d waves, workgroup barrier per segment>" % (

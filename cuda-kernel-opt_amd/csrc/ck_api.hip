@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <atomic>
 #include <mutex>
+#include <type_traits>
 
 #include "../../include/ckopt.h"
 #include "ck_common.h"
@@ -20,6 +21,7 @@ hipError_t launch_gemm_pcb_bf16(int tile, int segk, int cw, dim3 grid, dim3 bloc
 hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a);
 bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves);
+constexpr int STREAM_K_MULTIPLE_HOST = 64;  // K extent of one loop body of the straight-line kernel
 hipError_t launch_gemm_fused_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_fused_bf16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_matmul_shmem(int dtype, int tile, int accs, bool bt, dim3 grid, hipStream_t s, const SimtArgs& a);
@@ -37,6 +39,7 @@ std::atomic<int> g_prio_mode{0};
 std::atomic<int> g_producer_nap{0};
 std::atomic<int> g_tile_sync_barrier{0};
 std::atomic<int> g_straight_line{1};
+std::atomic<int> g_split_k{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
 
 constexpr int MAX_DEV = 64;
 std::mutex g_status_mutex;
@@ -72,6 +75,26 @@ __global__ void pad_rows_kernel(const unsigned short* __restrict__ src, unsigned
         o.x = v[0] | ((unsigned)v[1] << 16); o.y = v[2] | ((unsigned)v[3] << 16);
         o.z = v[4] | ((unsigned)v[5] << 16); o.w = v[6] | ((unsigned)v[7] << 16);
         *reinterpret_cast<uint4*>(dst + (long long)r * Kp + k0) = o;
+    }
+}
+
+// Second pass of a split-K product: D = alpha * (plane 0 + plane 1 + ...) + beta * C, the planes added in
+// slice order (the result does not depend on how the first pass was scheduled). One thread per element;
+// DT16 selects the 16-bit C/D forms.
+template <int OUT16, bool BF16>
+__global__ void splitk_reduce_kernel(const float* __restrict__ ws, int slices, long long count, const void* C, void* D, float alpha, float beta) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (long long)gridDim.x * blockDim.x) {
+        float sum = ws[i];
+        for (int s = 1; s < slices; ++s) sum += ws[(long long)s * count + i];
+        float v = alpha * sum;
+        if (OUT16) {
+            using O = ck::Out16<typename std::conditional<BF16, ck::bf16_tag, ck::f16_tag>::type>;
+            if (beta != 0.f) v += O::load(static_cast<const unsigned short*>(C)[i]) * beta;
+            static_cast<unsigned short*>(D)[i] = O::store(v);
+        } else {
+            if (beta != 0.f) v += static_cast<const float*>(C)[i] * beta;
+            static_cast<float*>(D)[i] = v;
+        }
     }
 }
 
@@ -149,9 +172,41 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     const size_t lds = (size_t)gemm_lds_bytes(t);
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
+    a.split_k = 1;
     if (g_straight_line.load() &&
         gemm_stream_applies(a, t.tile_dim, t.segment_dim_k, t.num_stages, t.num_producer_waves, t.num_consumer_waves)) {
-        e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a) : launch_gemm_stream_bf16(dim3(grid), s, a);
+        // Few tiles and a deep K (fewer tiles than half the CUs): cut K into slices so that every CU has
+        // an item, partial products into a stream-ordered workspace, one reduction pass. Needs whole
+        // XCD rounds of tiles (a multiple of 32) and slices of whole loop bodies.
+        int slices = 1;
+        const int want = g_split_k.load();
+        if (want != 0 && tiles % 32 == 0 && N % 4 == 0) {
+            int cand = want >= 2 ? want : (int)(t.num_cus / tiles);
+            if (cand > 16) cand = 16;
+            while (cand >= 2 && !(K % (cand * STREAM_K_MULTIPLE_HOST) == 0 && K / cand >= 1024)) --cand;
+            if (cand >= 2 && (want >= 2 || tiles * 2 <= t.num_cus)) slices = cand;
+        }
+        if (slices == 1) {
+            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a) : launch_gemm_stream_bf16(dim3(grid), s, a);
+        } else {
+            const long long count = (long long)M * N;
+            float* ws = nullptr;
+            if (hipMallocAsync((void**)&ws, (size_t)slices * count * sizeof(float), s) != hipSuccess || !ws) return CK_ERR_HIP;
+            GemmArgs p = a;
+            p.split_k = slices;
+            p.D = ws; p.C = nullptr; p.alpha = 1.f; p.beta = 0.f; p.out16 = 0; p.vec_store = 1;
+            const int64_t items = tiles * slices;
+            const int pgrid = (int)(items < t.num_cus ? items : t.num_cus);
+            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p) : launch_gemm_stream_bf16(dim3(pgrid), s, p);
+            if (e == hipSuccess) {
+                const unsigned blocks = (unsigned)((count + 255) / 256 < 65535 * 8 ? (count + 255) / 256 : 65535 * 8);
+                if (!out16) hipLaunchKernelGGL((splitk_reduce_kernel<0, false>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
+                else if (dtype == CK_DT_F16) hipLaunchKernelGGL((splitk_reduce_kernel<1, false>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
+                else hipLaunchKernelGGL((splitk_reduce_kernel<1, true>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
+                e = hipGetLastError();
+            }
+            if (hipFreeAsync(ws, s) != hipSuccess && e == hipSuccess) e = hipErrorUnknown;
+        }
     } else if (t.num_producer_waves == 0) {
         e = dtype == CK_DT_F16 ? launch_gemm_fused_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a)
                                : launch_gemm_fused_bf16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a);
@@ -340,6 +395,7 @@ int ckopt_set_option(int key, int value) {
         case 4: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_producer_nap.exchange(value);
         case 5: return g_tile_sync_barrier.exchange(value != 0);
         case 6: return g_straight_line.exchange(value != 0);
+        case 7: if (value < 0 || value > 16) return ck::CK_ERR_BAD_PARAM; return g_split_k.exchange(value);
         default: return ck::CK_ERR_BAD_PARAM;
     }
 }

@@ -4,6 +4,8 @@
 
 namespace ck {
 
+static_assert(STREAM_K_MULTIPLE == 64, "the host's slice rule assumes loop bodies of 64");
+
 template <typename DT>
 static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a) {
     auto kern = gemm_stream_kernel<DT>;
@@ -26,8 +28,7 @@ hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs
 // what the kernel assumes about a launch (the caller falls back to the general fused kernel otherwise)
 bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves) {
     return producer_waves == 0 && consumer_waves == 8 && tile_dim == STREAM_TILE && segment_dim_k == STREAM_SEGK &&
-           num_stages == STREAM_STAGES && a.M % STREAM_TILE == 0 && a.N % STREAM_TILE == 0 && a.K % STREAM_K_MULTIPLE == 0 &&
-           a.vec_store && a.swizzle;
+           num_stages == STREAM_STAGES && a.K % STREAM_K_MULTIPLE == 0 && a.swizzle;
 }
 
 }  // namespace ck

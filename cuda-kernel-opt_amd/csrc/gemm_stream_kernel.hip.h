@@ -1,9 +1,9 @@
 // The straight-line form of the fused (no dedicated producer waves) kernel for the shape the headline
-// sizes use: 256 x 256 tiles, eight waves, whole tiles only (M and N multiples of 256), K a multiple
-// of 64, and a ring of five 32-deep K segments ("quarters", 32 KiB each) - all of the CU's LDS. With
-// those fixed the loop body is two k-steps, the loader runs exactly two bodies ahead of the
-// multiplier, and every wait is an immediate - no mode flags, no wait ladder, no per-segment
-// bookkeeping between the MFMAs.
+// sizes use: 256 x 256 tiles, eight waves, K a multiple of 64 (M and N are free: ragged tiles read
+// zeros past the edge and store element by element), and a ring of five 32-deep K segments
+// ("quarters", 32 KiB each) - all of the CU's LDS. With those fixed the loop body is two k-steps,
+// the loader runs exactly two bodies ahead of the multiplier, and every wait is an immediate - no
+// mode flags, no wait ladder, no per-segment bookkeeping between the MFMAs.
 //
 // Why five quarters and "pair fetch": a 32-deep segment is 64 bytes of each operand row, half a
 // cache line. Fetching the halves in different k-steps makes the L1 ask the L2 for every line twice
@@ -35,6 +35,15 @@
 
 #include "gemm_fused_kernel.hip.h"
 
+// schedule constants (tuning builds override them)
+#ifndef CK_STREAM_PRE
+#define CK_STREAM_PRE 1
+#endif
+#ifndef CK_STREAM_LOAD_COL_0
+#define CK_STREAM_LOAD_COL_0 3
+#define CK_STREAM_LOAD_COL_1 6
+#endif
+
 namespace ck {
 
 constexpr int STREAM_TILE = 256;
@@ -52,6 +61,10 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     constexpr int QB = 2 * OPB;              // one quarter
     constexpr int LPB = 8;                   // loads per wave and body: (A, Bt) x (rows w, w + 8) x (two halves)
     constexpr int EPILOGUE_STORES = WTR * WTC;
+    constexpr int PRE = CK_STREAM_PRE;               // columns of MFMAs in front of the barrier
+    constexpr int LOAD_COL_0 = CK_STREAM_LOAD_COL_0;  // columns behind which a k-step's two load pairs are issued
+    constexpr int LOAD_COL_1 = CK_STREAM_LOAD_COL_1;
+    static_assert(PRE >= 1 && (WTC - PRE) * 2 >= WTR + WTC && LOAD_COL_0 >= PRE && LOAD_COL_1 > LOAD_COL_0 && LOAD_COL_1 < WTC, "schedule");
     static_assert(LPB + EPILOGUE_STORES < 64, "the wait immediates must fit the 6-bit counter");
     static_assert(STREAM_LDS_BYTES <= LDS_BYTES_PER_CU, "the ring is all of the LDS");
 
@@ -63,9 +76,21 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 
     const int grid = gridDim.x;
     const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
-    const int total_tiles = g.tiles_m * g.tiles_n;
-    const int my_tiles = slot < total_tiles ? (total_tiles - slot + grid - 1) / grid : 0;
-    const int nb = g.K / STREAM_K_MULTIPLE;  // loop bodies per tile
+    // Work items: one per (tile, K slice). Item numbers are dealt like tile counts (slot, slot + grid, ...);
+    // 32 consecutive items - what one XCD runs at a time - are 32 consecutive tile counts of ONE slice, so
+    // they share operand panels in that XCD's L2 exactly as whole tiles do. Without split-K an item is
+    // a tile count.
+    const int S = g.split_k;
+    const int total_items = g.tiles_m * g.tiles_n * S;
+    const int my_tiles = slot < total_items ? (total_items - slot + grid - 1) / grid : 0;
+    const int kslice = g.K / S;                  // the host makes this a multiple of one loop body
+    const uint32_t kslice_bytes = (uint32_t)kslice * 2u;
+    const int nb = kslice / STREAM_K_MULTIPLE;   // loop bodies per item
+    auto item_tile = [&](int64_t item, int& slice) __attribute__((always_inline)) {
+        const int64_t chunk = item / 32;
+        slice = (int)(chunk % S);
+        return (chunk / S) * 32 + item % 32;
+    };
 
     // ---- loader ------------------------------------------------------------------------------------
     // A wave load covers 16 rows x 64 bytes of an operand quarter; wave w issues the loads of rows
@@ -74,24 +99,30 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     // block only).
     const uint32_t pitch32 = (uint32_t)g.K * 2u;
     const int lane_row = lane / 4, lane_slot = lane % 4;
-    const uint32_t loff = (uint32_t)lane_row * pitch32 + (uint32_t)swizzle_slot(lane_row, lane_slot, 4, 1) * CHUNK_BYTES;
+    // The row part of the address goes through the range-checked per-lane offset (rows past the edge
+    // of a ragged tile lie outside the descriptor and read as zeros), the k part through the
+    // unchecked scalar offset.
+    const uint32_t loff_lo = (uint32_t)(wave * 16 + lane_row) * pitch32 + (uint32_t)swizzle_slot(lane_row, lane_slot, 4, 1) * CHUNK_BYTES;
+    const uint32_t loff_hi = loff_lo + 8u * 16u * pitch32;   // rows 16(w+8)..
     const uint32_t dst_w = ring_base + (uint32_t)wave * 1024u;
-    const uint32_t goff_w = (uint32_t)wave * 16u * pitch32;
-    const uint32_t goff_hi = 8u * 16u * pitch32;   // rows 16(w+8).. relative to rows 16w..
-    const uint32_t nrec = (uint32_t)TILE * pitch32;
     i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // empty descriptors: loads read zeros
     uint32_t l_koff = 0;  // byte offset along K of the body being loaded
     int l_tile = 0;       // index (in this workgroup's list) of the tile being loaded
     auto loader_open_tile = [&]() __attribute__((always_inline)) {
         if (l_tile < my_tiles) {
+            int slice = 0;
+            const int64_t tc = item_tile(slot + (int64_t)l_tile * grid, slice);
 #if defined(CK_PROBE_SAME_TILE)  // measurement build only: every workgroup loads the operands of tile (0, 0)
             const TileRC rc{0, 0};
 #else
-            const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, slot + (int64_t)l_tile * grid);
+            const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
 #endif
             const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE);
-            rsrc_a = make_rsrc((const char*)g.A + (int64_t)row_a * pitch32, nrec);
-            rsrc_b = make_rsrc((const char*)g.Bt + (int64_t)row_b * pitch32, nrec);
+            const int ra = g.M - row_a < TILE ? g.M - row_a : TILE, rb = g.N - row_b < TILE ? g.N - row_b : TILE;
+            const int64_t k0 = (int64_t)slice * kslice_bytes;  // the slice starts k0 bytes into every row
+            // (the descriptor's extent is counted from the shifted base: the last row ends k0 bytes early)
+            rsrc_a = make_rsrc((const char*)g.A + (int64_t)row_a * pitch32 + k0, (uint32_t)ra * pitch32 - (uint32_t)k0);
+            rsrc_b = make_rsrc((const char*)g.Bt + (int64_t)row_b * pitch32 + k0, (uint32_t)rb * pitch32 - (uint32_t)k0);
         } else {
             rsrc_a[2] = 0;  // past the last tile: nothing is fetched (the ring receives zeros nobody reads)
             rsrc_b[2] = 0;
@@ -99,7 +130,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     };
     auto loader_advance = [&]() __attribute__((always_inline)) {
         l_koff += STREAM_K_MULTIPLE * 2;
-        if (l_koff == pitch32) {
+        if (l_koff == kslice_bytes) {
             l_koff = 0;
             ++l_tile;
             loader_open_tile();
@@ -112,9 +143,8 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         constexpr bool IS_A = P < 2;
         constexpr int HI = P % 2;
         const uint32_t dst = dst_w + (uint32_t)((IS_A ? 0 : OPB) + HI * 8 * 1024);
-        const uint32_t soff = goff_w + (HI ? goff_hi : 0u) + l_koff;
-        dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_lo, loff, soff);
-        dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_hi, loff, soff + (uint32_t)(STREAM_SEGK * 2));
+        dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_lo, HI ? loff_hi : loff_lo, l_koff);
+        dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_hi, HI ? loff_hi : loff_lo, l_koff + (uint32_t)(STREAM_SEGK * 2));
     };
 
     // ---- multiplier --------------------------------------------------------------------------------
@@ -167,16 +197,18 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #endif
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < WTR; ++i) acc[i][0] = MfmaOp<DT>::run(fb[P][0], fa[P][i], acc[i][0]);
+        for (int j = 0; j < PRE; ++j)
+#pragma unroll
+            for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         wg_barrier();
         __builtin_amdgcn_sched_barrier(0);
         const uint32_t pa = a_lane + qn, pb = b_lane + qn;
 #pragma unroll
-        for (int j = 1; j < WTC; ++j) {
+        for (int j = PRE; j < WTC; ++j) {
 #pragma unroll
             for (int q = 0; q < 2; ++q) {
-                const int f = (j - 1) * 2 + q;
+                const int f = (j - PRE) * 2 + q;
                 if (f < WTR) fa[1 - P][f] = *(const CK_LDS u32x4*)(uintptr_t)(pa + (uint32_t)(f * 16 * RB));
                 else if (f < WTR + WTC) fb[1 - P][f - WTR] = *(const CK_LDS u32x4*)(uintptr_t)(pb + (uint32_t)((f - WTR) * 16 * RB));
             }
@@ -184,8 +216,8 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             // this k-step's share of the loads, one pair behind every third column: the pairs of A in the
             // even k-step, those of Bt in the odd one (a wave stalls on back-to-back loads, and both waves
             // of a SIMD run in step)
-            if (j == 3) issue_pair(std::integral_constant<int, 2 * P>{}, q4, q0);
-            if (j == 6) issue_pair(std::integral_constant<int, 2 * P + 1>{}, q4, q0);
+            if (j == LOAD_COL_0) issue_pair(std::integral_constant<int, 2 * P>{}, q4, q0);
+            if (j == LOAD_COL_1) issue_pair(std::integral_constant<int, 2 * P + 1>{}, q4, q0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
@@ -237,9 +269,14 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             const unsigned long long te0 = clock64();
 #endif
             // D = alpha * acc + beta * C straight from the accumulators
-            const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, slot + (int64_t)t * grid);
+            int slice = 0;
+            const int64_t tc = item_tile(slot + (int64_t)t * grid, slice);
+            const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
+            GemmArgs go = g;  // a K slice writes its own plane of the workspace D points at
+            go.D = g.D + (size_t)slice * ((size_t)g.M * g.N);
             const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
             const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
+            const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
 #pragma unroll
             for (int i = 0; i < WTR; ++i) {
 #pragma unroll
@@ -247,7 +284,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #if defined(CK_PROBE_NO_EPILOGUE)  // measurement build only: nothing is written (except by a workgroup that never exists)
                     if (blockIdx.x == 0x7fffffff)
 #endif
-                    epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], true);
+                    epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
                     acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
                 }
             }
@@ -256,7 +293,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #endif
             // (set through asm so that the flag stays one opaque scalar register: otherwise the compiler
             // peels the loop around its known values)
-            asm volatile("s_mov_b32 %0, %1" : "=s"(stores_in_flight) : "s"(count_stores));
+            asm volatile("s_mov_b32 %0, %1" : "=s"(stores_in_flight) : "s"(interior ? count_stores : 0u));
         }
         // the loads issued past the last tile fetch nothing, but they still write the ring
         wait_vmcnt_imm<0>();

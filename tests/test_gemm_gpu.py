@@ -493,6 +493,10 @@ def _straight_line_tuning(ck, cus=256, group=4):
     (1024, 1024, 192, 5, 4),
     (1024, 1280, 1152, 7, 3),    # group size that does not divide the tile rows
     (2048, 2048, 1024, 256, 4),
+    (300, 260, 128, 256, 4),     # ragged tiles: rows past the edge read as zeros, element-wise stores
+    (777, 515, 192, 3, 4),       # N not a multiple of 4: no vector stores anywhere
+    (100, 50, 64, 256, 4),
+    (1279, 1025, 320, 7, 3),
 ])
 def test_straight_line_kernel_bit_exact(ck, M, N, K, cus, group):
     t = _straight_line_tuning(ck, cus, group)
@@ -541,3 +545,43 @@ def test_straight_line_kernel_headline_size_properties(ck):
     eye[np.arange(N), (np.arange(N) * 5 + 3) % K] = 1.0
     d = G.run_gemm(ck, ck.DT_F16, a, eye, t=t)
     assert np.array_equal(d, a[:, (np.arange(N) * 5 + 3) % K].astype(np.float32))
+
+
+@pytest.mark.parametrize("M,N,K,slices,cus,dt_name", [
+    (2048, 1024, 4096, 4, 256, "f16"),
+    (2048, 1024, 4096, 2, 5, "f16"),      # several items per workgroup, slices of different tiles in turn
+    (2048, 1024, 8192, 8, 256, "bf16"),
+    (2048, 2048, 4096, 1, 256, "f16"),    # automatic: 64 tiles on 256 CUs
+    (2000, 1020, 4096, 4, 256, "f16"),    # ragged tiles
+])
+def test_split_k_bit_exact(ck, M, N, K, slices, cus, dt_name):
+    dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16
+    t = _straight_line_tuning(ck, cus)
+    a = ck.fill_int(dt, (M, K), 95, 0, -2, 2)
+    bt = ck.fill_int(dt, (N, K), 95, 1, -2, 2)
+    c = ck.fill_int(ck.DT_F32, (M, N), 95, 2, -3, 3)
+    want = (2.0 * (G.as_f64(dt == ck.DT_BF16, a) @ G.as_f64(dt == ck.DT_BF16, bt).T) - c.astype(np.float64)).astype(np.float32)
+    prev = ck.set_option(ck.OPT_SPLIT_K, slices)
+    try:
+        got = G.run_gemm(ck, dt, a, bt, c, 2.0, -1.0, t=t)
+    finally:
+        ck.set_option(ck.OPT_SPLIT_K, prev)
+    assert np.array_equal(got, want)
+
+
+def test_split_k_against_the_oracle_and_the_single_pass(ck, oracle):
+    # uniform data: the sliced sum differs from the single pass in rounding only
+    M, N, K = 2048, 1024, 4096
+    t = _straight_line_tuning(ck)
+    a = ck.fill_uniform(ck.DT_F16, (M, K), 96, 0)
+    bt = ck.fill_uniform(ck.DT_F16, (N, K), 96, 1)
+    ref = oracle.gemm(oracle.DT_F16, a, bt, None, 1.0, 0.0)
+    out = {}
+    for slices in (0, 4):
+        prev = ck.set_option(ck.OPT_SPLIT_K, slices)
+        try:
+            out[slices] = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+        finally:
+            ck.set_option(ck.OPT_SPLIT_K, prev)
+        assert_close(oracle, ref, out[slices])
+    assert_close(oracle, out[0], out[4], rtol=1e-4)

@@ -193,3 +193,14 @@ def test_normal_and_int_generators(ck):
     assert set(np.unique(h.astype(np.int32))) == {-2, -1, 0, 1, 2}
     c = ck.fill_constant(ck.DT_BF16, (8,), 10.0)
     assert np.all(c == 0x4120)
+
+
+def test_option_keys_reject_values_outside_their_range(ck):
+    # process-wide switches: a bad value changes nothing and reports the error
+    for key, bad in ((ck.OPT_NUM_XCD, 0), (ck.OPT_PRIO_MODE, 3), (ck.OPT_PRODUCER_NAP, -1), (ck.OPT_SPLIT_K, 17), (99, 1)):
+        with pytest.raises(ck.CkoptError):
+            ck.set_option(key, bad)
+    prev = ck.set_option(ck.OPT_SPLIT_K, 0)
+    assert ck.set_option(ck.OPT_SPLIT_K, prev) == 0
+    prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
+    assert ck.set_option(ck.OPT_STRAIGHT_LINE, prev) == 0
