@@ -143,8 +143,8 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
             o.x = (uint32_t)Out16<DT>::store(v[0]) | ((uint32_t)Out16<DT>::store(v[1]) << 16);
             o.y = (uint32_t)Out16<DT>::store(v[2]) | ((uint32_t)Out16<DT>::store(v[3]) << 16);
 #if defined(CK_NT_STORE)
-            __builtin_nontemporal_store(o.x, (uint32_t*)(d16 + off));
-            __builtin_nontemporal_store(o.y, (uint32_t*)(d16 + off) + 1);
+            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+            __builtin_nontemporal_store(u32x2{o.x, o.y}, (u32x2*)(d16 + off));
 #else
             *(uint2*)(d16 + off) = o;
 #endif

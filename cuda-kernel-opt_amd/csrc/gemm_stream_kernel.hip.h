@@ -277,17 +277,55 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
             const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
             const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
-#pragma unroll
-            for (int i = 0; i < WTR; ++i) {
-#pragma unroll
-                for (int j = 0; j < WTC; ++j) {
 #if defined(CK_PROBE_NO_EPILOGUE)  // measurement build only: nothing is written (except by a workgroup that never exists)
-                    if (blockIdx.x == 0x7fffffff)
+            if (blockIdx.x == 0x7fffffff)
 #endif
-                    epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
-                    acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#if defined(CK_STREAM_BLOCK_STORES)  // tuning builds: one store per accumulator block (half lines)
+            if (false) {
+#else
+            if (interior && !g.out16) {
+#endif
+                // Whole 128-byte lines per store: an accumulator block gives a row 64 bytes (4 lanes x 16),
+                // and the write path's cost is per request, not per byte. Two neighbouring blocks are
+                // exchanged between lanes so that 8 lanes hold the 32 consecutive floats of one row:
+                // store t (0, 1) of a pair writes rows 8t .. 8t+7, lane L the piece L % 8 of row L / 8,
+                // which sits in lane (8t + L / 8) + 16 * (piece % 4) of block piece / 4.
+                const int piece = lane & 7;
+                const int src0 = ((lane >> 3) + 16 * (piece & 3)) * 4;  // byte address of the source lane, t = 0
+                const bool second = piece >= 4;
+                const int64_t row0 = (int64_t)(rc.row * TILE + R * WTR * 16 + (lane >> 3));
+                const int col0 = rc.col * TILE + Cc * WTC * 16 + piece * 4;
+                const float alpha = g.alpha, beta = g.beta;
+#pragma unroll
+                for (int i = 0; i < WTR; ++i) {
+#pragma unroll
+                    for (int j = 0; j < WTC; j += 2) {
+#pragma unroll
+                        for (int tt = 0; tt < 2; ++tt) {
+                            f32x4 v;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const float x0 = acc[i][j][e], x1 = acc[i][j + 1][e];
+                                const int a0 = __builtin_amdgcn_ds_bpermute(src0 + tt * 32, __float_as_int(x0));
+                                const int a1 = __builtin_amdgcn_ds_bpermute(src0 + tt * 32, __float_as_int(x1));
+                                v[e] = __int_as_float(second ? a1 : a0) * alpha;
+                            }
+                            const int64_t off = (row0 + i * 16 + tt * 8) * g.N + (col0 + j * 16);
+                            if (beta != 0.f) v += *(const f32x4*)(go.C + off) * beta;
+                            __builtin_nontemporal_store(v, (f32x4*)(go.D + off));
+                        }
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int i = 0; i < WTR; ++i)
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j) epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
             }
+#pragma unroll
+            for (int i = 0; i < WTR; ++i)
+#pragma unroll
+                for (int j = 0; j < WTC; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #if defined(CK_PROBE_TIMING)
             t_epi += clock64() - te0;
 #endif
