@@ -362,3 +362,140 @@ class _AlwaysEmptyView(list):
     """In-flight queue whose contents the landing check cannot see (iteration yields nothing)."""
     def __iter__(self):
         return iter(())
+
+
+# ---- the straight-line kernel: five quarters, pair fetch, counted waits --------------------------------
+class StreamModel:
+    """Waves of the straight-line 256 x 256 kernel, restated from its schedule. Every wave keeps one queue
+    of vector memory operations that complete in issue order (loads and the epilogue's stores alike) and
+    waits with `outstanding <= immediate`, exactly as `s_waitcnt vmcnt` does. Loop body = even and odd
+    k-step of a work item's K range; in the even k-step a wave issues its two A load pairs of the body two
+    ahead, in the odd one the two Bt pairs; each pair is two loads (the halves of a line) into quarters
+    (j + 4) % 5 and j % 5 of the even k-step j. The odd k-step waits with immediate 4 (+ 32 behind an
+    epilogue without C reads); every k-step has one barrier, behind it the fragments of the next k-step
+    are read. Checked: a read finds every wave's share of the expected k-step in the quarter (nothing
+    late, nothing overwritten early), and all waves finish."""
+
+    LOADS_PER_KSTEP = 4
+    STORES = 32
+
+    def __init__(self, waves, bodies_per_item, items, rng, imm=4, imm_stores=36, count_stores=True, completion_rate=0.35, slow_wave=None):
+        self.n, self.nb, self.items, self.rng = waves, bodies_per_item, items, rng
+        self.completion_rate = completion_rate                       # how eagerly the memory system answers
+        self.slow_wave = slow_wave                                   # a wave whose operations complete 50 times more rarely
+        self.imm, self.imm_stores, self.count_stores = imm, imm_stores, count_stores
+        self.total = 2 * bodies_per_item * items                     # k-steps in the stream
+        # per quarter and wave, per load of a k-step (A rows 16w.., A rows 16(w+8).., Bt likewise): k-step it holds
+        self.holds = [[[-1, -1, -1, -1] for _ in range(waves)] for _ in range(5)]
+        self.queue = [[] for _ in range(waves)]                       # per wave: FIFO of ops
+        self.arrived, self.generation = 0, 0
+        self.errors = []
+
+    def complete_some(self):
+        w = self.rng.randrange(self.n)
+        if w == self.slow_wave and self.rng.random() > 0.02:
+            return
+        if self.queue[w]:
+            op = self.queue[w].pop(0)
+            if op[0] == "load":
+                _, quarter, slot, kstep = op
+                self.holds[quarter][w][slot] = kstep
+
+    def read(self, quarter, kstep):
+        for w in range(self.n):
+            if self.holds[quarter][w] != [kstep] * 4:
+                self.errors.append("k-step %d read from quarter %d: wave %d's share holds %s" % (kstep, quarter, w, self.holds[quarter][w]))
+
+    def issue_pairs(self, w, operand, even_kstep, body_kstep):
+        # two pairs = four loads of the body whose even k-step is body_kstep, issued in (or before) the body
+        # of even k-step even_kstep, which fixes the quarters: lo halves -> body_kstep % 5, hi halves -> + 1
+        for pair in range(2):
+            for half in range(2):
+                k = body_kstep + half
+                self.queue[w].append(("load", k % 5, 2 * operand + pair, k if k < self.total else -2))
+
+    def wave(self, w):
+        def barrier():
+            gen = self.generation
+            self.arrived += 1
+            if self.arrived == self.n:
+                self.arrived = 0
+                self.generation += 1
+            while self.generation == gen:
+                yield
+        def wait(imm):
+            while len(self.queue[w]) > imm:
+                yield
+        # prologue: both operands of bodies 0 and 1, then k-step 0 in registers
+        for body in (0, 1):
+            for operand in (0, 1):
+                self.issue_pairs(w, operand, 0, 2 * body)
+        yield from wait(8)
+        yield from barrier()
+        self.read(0, 0)
+        stores_in_flight = False
+        for j in range(0, self.total, 2):
+            # even k-step j
+            yield from barrier()
+            yield
+            self.read((j + 1) % 5, j + 1)
+            self.issue_pairs(w, 0, j, j + 4)
+            yield
+            # odd k-step j + 1
+            yield from wait(self.imm_stores if stores_in_flight else self.imm)
+            yield from barrier()
+            yield
+            if j + 2 < self.total:
+                self.read((j + 2) % 5, j + 2)
+            self.issue_pairs(w, 1, j, j + 4)
+            stores_in_flight = False
+            if (j + 2) % (2 * self.nb) == 0:                          # the item ends: epilogue
+                for _ in range(self.STORES):
+                    self.queue[w].append(("store",))
+                stores_in_flight = self.count_stores
+            yield
+
+    def run(self):
+        gens = [self.wave(w) for w in range(self.n)]
+        alive = list(range(self.n))
+        steps = 0
+        while alive:
+            steps += 1
+            if steps > 2000000:
+                return "deadlock"
+            if self.rng.random() < self.completion_rate:
+                self.complete_some()
+                continue
+            i = self.rng.choice(alive)
+            try:
+                next(gens[i])
+            except StopIteration:
+                alive.remove(i)
+        return None
+
+
+@pytest.mark.parametrize("bodies,items", [(1, 1), (1, 5), (2, 3), (3, 2), (7, 2), (16, 1)])
+def test_stream_schedule(bodies, items):
+    for seed, rate, slow in ((0, 0.35, None), (1, 0.35, 3), (2, 0.05, None), (3, 0.05, 6)):   # eager, sluggish, one starved wave
+        m = StreamModel(8, bodies, items, random.Random(1000 * bodies + 10 * items + seed), completion_rate=rate, slow_wave=slow)
+        assert m.run() is None
+        assert not m.errors, m.errors[:3]
+    # with C reads in the epilogue the kernel does not count the stores: the stricter immediate is also safe
+    m = StreamModel(8, bodies, items, random.Random(7), count_stores=False)
+    assert m.run() is None and not m.errors
+
+
+def test_stream_model_detects_wrong_immediates():
+    # sanity of the checker: one operation too many allowed in flight, with and without the stores
+    caught = 0
+    for seed in range(20):
+        m = StreamModel(8, 3, 3, random.Random(seed), imm=5, imm_stores=37, completion_rate=0.3, slow_wave=seed % 8)
+        m.run()
+        caught += bool(m.errors)
+    assert caught > 0
+    caught = 0
+    for seed in range(20):
+        m = StreamModel(8, 1, 6, random.Random(seed), imm=4, imm_stores=37, completion_rate=0.3, slow_wave=seed % 8)
+        m.run()
+        caught += bool(m.errors)
+    assert caught > 0
