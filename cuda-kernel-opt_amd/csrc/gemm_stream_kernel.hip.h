@@ -219,8 +219,13 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             if (j == LOAD_COL_0) issue_pair(std::integral_constant<int, 2 * P>{}, q4, q0);
             if (j == LOAD_COL_1) issue_pair(std::integral_constant<int, 2 * P + 1>{}, q4, q0);
             __builtin_amdgcn_sched_barrier(0);
+            // every other column runs its rows backwards: one operand register changes per MFMA instead of
+            // two at the column boundaries (+0.7 % on random operands, where the device is power-limited)
 #pragma unroll
-            for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
+            for (int ii = 0; ii < WTR; ++ii) {
+                const int i = (j & 1) ? WTR - 1 - ii : ii;
+                acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
