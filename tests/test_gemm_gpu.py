@@ -322,8 +322,9 @@ def test_config4_long_k_shift_sync_regime(ck, oracle):
     M = N = 2048
     K = 32768
     fill = lambda s, shape: ck.fill_normal(ck.DT_F16, shape, 0xC0FFEE04, s, 0.0, 0.1)
+    # the last tuple is the straight-line kernel: 64 tiles of 256 x 256, K cut into 4 slices + reduction pass
     for t in (make_tuning(ck, 128, 64, 4, 4, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 4, 2),
-              make_tuning(ck, 128, 64, 4, 4, 8, "acc", 1, 3)):
+              make_tuning(ck, 128, 64, 4, 4, 8, "acc", 1, 3), make_tuning(ck, 256, 32, 5, 0, 8)):
         full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t, fill, rows=(0, 1024))
 
 
@@ -363,15 +364,17 @@ def test_config5_bf16_6143x4097x3071(ck, oracle):
     # oracle within the stated tolerance, and the row-sum identity over the whole result
     M, N, K = 6143, 4097, 3071
     fill = lambda s, shape: ck.fill_uniform(ck.DT_BF16, shape, 0xC0FFEE05, s)
-    for t in (make_tuning(ck, 256, 64, 2, 2, 8), make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 2, 1)):
+    for t in (make_tuning(ck, 256, 64, 2, 2, 8), make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 2, 1),
+              make_tuning(ck, 256, 32, 5, 0, 8)):
         full_size_check(ck, oracle, ck.DT_BF16, oracle.DT_BF16, M, N, K, t, fill, rows=(0, 3000, M - 8))
     # exact at full size on small integers
     a = ck.fill_int(ck.DT_BF16, (M, K), 0xC0FFEE05, 2, -1, 1)
     bt = ck.fill_int(ck.DT_BF16, (N, K), 0xC0FFEE05, 3, -1, 1)
-    d = G.run_gemm(ck, ck.DT_BF16, a, bt, t=make_tuning(ck, 256, 64, 2, 2, 8))
     ai, bi = G.as_f64(True, a).astype(np.int64), G.as_f64(True, bt).astype(np.int64)
-    assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
-    assert np.array_equal(d[M - 1], (ai[M - 1] @ bi.T).astype(np.float32))
+    for t in (make_tuning(ck, 256, 64, 2, 2, 8), make_tuning(ck, 256, 32, 5, 0, 8)):
+        d = G.run_gemm(ck, ck.DT_BF16, a, bt, t=t)
+        assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
+        assert np.array_equal(d[M - 1], (ai[M - 1] @ bi.T).astype(np.float32))
 
 
 def test_fused_variant_full_size(ck, oracle):
