@@ -18,8 +18,8 @@ CK_DECL_GEMM(launch_gemm_pc_bf16_m0) CK_DECL_GEMM(launch_gemm_pc_bf16_m1) CK_DEC
 #undef CK_DECL_GEMM
 hipError_t launch_gemm_pcb_f16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_pcb_bf16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
-hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a);
-hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a);
+hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep);
+hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep);
 bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves);
 constexpr int STREAM_K_MULTIPLE_HOST = 64;  // K extent of one loop body of the straight-line kernel
 hipError_t launch_gemm_fused_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
@@ -39,7 +39,8 @@ std::atomic<int> g_prio_mode{0};
 std::atomic<int> g_producer_nap{0};
 std::atomic<int> g_tile_sync_barrier{0};
 std::atomic<int> g_straight_line{1};
-std::atomic<int> g_split_k{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
+std::atomic<int> g_split_k{1};
+std::atomic<int> g_barrier_every_kstep{0};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
 
 constexpr int MAX_DEV = 64;
 std::mutex g_status_mutex;
@@ -179,6 +180,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         // an item, partial products into a stream-ordered workspace, one reduction pass. Needs whole
         // XCD rounds of tiles (a multiple of 32) and slices of whole loop bodies.
         int slices = 1;
+        const bool bek = g_barrier_every_kstep.load() != 0;
         const int want = g_split_k.load();
         if (want != 0 && tiles % 32 == 0 && N % 4 == 0) {
             int cand = want >= 2 ? want : (int)(t.num_cus / tiles);
@@ -187,7 +189,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             if (cand >= 2 && (want >= 2 || tiles * 2 <= t.num_cus)) slices = cand;
         }
         if (slices == 1) {
-            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a) : launch_gemm_stream_bf16(dim3(grid), s, a);
+            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a, bek) : launch_gemm_stream_bf16(dim3(grid), s, a, bek);
         } else {
             const long long count = (long long)M * N;
             float* ws = nullptr;
@@ -197,7 +199,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             p.D = ws; p.C = nullptr; p.alpha = 1.f; p.beta = 0.f; p.out16 = 0; p.vec_store = 1;
             const int64_t items = tiles * slices;
             const int pgrid = (int)(items < t.num_cus ? items : t.num_cus);
-            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p) : launch_gemm_stream_bf16(dim3(pgrid), s, p);
+            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p, bek) : launch_gemm_stream_bf16(dim3(pgrid), s, p, bek);
             if (e == hipSuccess) {
                 const unsigned blocks = (unsigned)((count + 255) / 256 < 65535 * 8 ? (count + 255) / 256 : 65535 * 8);
                 if (!out16) hipLaunchKernelGGL((splitk_reduce_kernel<0, false>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
@@ -396,6 +398,7 @@ int ckopt_set_option(int key, int value) {
         case 5: return g_tile_sync_barrier.exchange(value != 0);
         case 6: return g_straight_line.exchange(value != 0);
         case 7: if (value < 0 || value > 16) return ck::CK_ERR_BAD_PARAM; return g_split_k.exchange(value);
+        case 8: return g_barrier_every_kstep.exchange(value != 0);
         default: return ck::CK_ERR_BAD_PARAM;
     }
 }

@@ -6,9 +6,9 @@ namespace ck {
 
 static_assert(STREAM_K_MULTIPLE == 64, "the host's slice rule assumes loop bodies of 64");
 
-template <typename DT>
+template <typename DT, bool ODD_ONLY>
 static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a) {
-    auto kern = gemm_stream_kernel<DT>;
+    auto kern = gemm_stream_kernel<DT, ODD_ONLY>;
     static bool opted[64] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -22,8 +22,13 @@ static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a
     return hipGetLastError();
 }
 
-hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a) { return stream_launch<f16_tag>(grid, stream, a); }
-hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a) { return stream_launch<bf16_tag>(grid, stream, a); }
+// barrier_every_kstep selects the schedule with a barrier in both k-steps of a loop body
+hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep) {
+    return barrier_every_kstep ? stream_launch<f16_tag, false>(grid, stream, a) : stream_launch<f16_tag, true>(grid, stream, a);
+}
+hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep) {
+    return barrier_every_kstep ? stream_launch<bf16_tag, false>(grid, stream, a) : stream_launch<bf16_tag, true>(grid, stream, a);
+}
 
 // what the kernel assumes about a launch (the caller falls back to the general fused kernel otherwise)
 bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves) {

@@ -21,6 +21,11 @@
 //     fragments in registers; own loads of k-steps j+2, j+3 landed (the four just issued may fly);
 //     first column; barrier -> quarters q+2, q+3 complete; 7 columns, fragments of j+2 from q+2 and
 //     the four loads of Bt for k-steps j+4 and j+5
+// ODD_ONLY (the default) drops the even k-step's barrier: all four pairs of a body are then issued in the
+// odd k-step, behind its barrier (by then quarter q is free as well), and the odd k-step waits for
+// all of the wave's loads. That leaves the loads two k-steps instead of three and bunches them, which
+// costs 3 % when the clock is fixed (all-zero operands) - and gains 1-1.5 % on random operands, where
+// the device is power-limited and fewer synchronisation points let it hold a higher clock.
 // The stream of k-steps runs across the tiles of the persistent workgroup; the loader moves to the
 // next tile two bodies before the multiplier does, so its first quarters are in flight while the
 // current tile is finished and written out.
@@ -52,7 +57,7 @@ constexpr int STREAM_STAGES = 5;
 constexpr int STREAM_K_MULTIPLE = 2 * STREAM_SEGK;  // one loop body
 constexpr int STREAM_LDS_BYTES = STREAM_STAGES * 2 * STREAM_TILE * STREAM_SEGK * 2;
 
-template <typename DT>
+template <typename DT, bool ODD_ONLY>
 __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     constexpr int TILE = STREAM_TILE, NQ = STREAM_STAGES;
     constexpr int WTR = 4, WTC = 8;          // 16 x 16 blocks per wave tile (64 x 128)
@@ -191,7 +196,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             // and fragment registers live across them.)
             asm volatile("s_cmp_lg_u32 %0, 0\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(%1)\n1:\n\ts_waitcnt vmcnt(%2)"
                          :
-                         : "s"(stores_in_flight), "n"(LPB / 2), "n"(LPB / 2 + EPILOGUE_STORES)
+                         : "s"(stores_in_flight), "n"(ODD_ONLY ? 0 : LPB / 2), "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES)
                          : "memory", "scc");
         }
 #endif
@@ -201,7 +206,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
             for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
-        wg_barrier();
+        if constexpr (!ODD_ONLY || P == 1) wg_barrier();
         __builtin_amdgcn_sched_barrier(0);
         const uint32_t pa = a_lane + qn, pb = b_lane + qn;
 #pragma unroll
@@ -213,11 +218,21 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                 else if (f < WTR + WTC) fb[1 - P][f - WTR] = *(const CK_LDS u32x4*)(uintptr_t)(pb + (uint32_t)((f - WTR) * 16 * RB));
             }
             __builtin_amdgcn_sched_barrier(0);
-            // this k-step's share of the loads, one pair behind every third column: the pairs of A in the
-            // even k-step, those of Bt in the odd one (a wave stalls on back-to-back loads, and both waves
-            // of a SIMD run in step)
-            if (j == LOAD_COL_0) issue_pair(std::integral_constant<int, 2 * P>{}, q4, q0);
-            if (j == LOAD_COL_1) issue_pair(std::integral_constant<int, 2 * P + 1>{}, q4, q0);
+            // this k-step's share of the loads, spread over the columns (a wave stalls on back-to-back
+            // loads, and both waves of a SIMD run in step); with a barrier in every k-step: the pairs of
+            // A in the even k-step, those of Bt in the odd one
+            if constexpr (ODD_ONLY) {
+                // all four pairs in the odd k-step, behind its barrier (the only one of the body)
+                if constexpr (P == 1) {
+                    if (j == 2) issue_pair(std::integral_constant<int, 0>{}, q4, q0);
+                    if (j == 4) issue_pair(std::integral_constant<int, 1>{}, q4, q0);
+                    if (j == 6) issue_pair(std::integral_constant<int, 2>{}, q4, q0);
+                    if (j == 7) issue_pair(std::integral_constant<int, 3>{}, q4, q0);
+                }
+            } else {
+                if (j == LOAD_COL_0) issue_pair(std::integral_constant<int, 2 * P>{}, q4, q0);
+                if (j == LOAD_COL_1) issue_pair(std::integral_constant<int, 2 * P + 1>{}, q4, q0);
+            }
             __builtin_amdgcn_sched_barrier(0);
             // every other column runs its rows backwards: one operand register changes per MFMA instead of
             // two at the column boundaries (+0.7 % on random operands, where the device is power-limited)

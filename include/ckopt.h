@@ -156,6 +156,9 @@ int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, do
  *        (hipMallocAsync, slices * M * N * 4 bytes) and a second kernel adds them in slice order and applies
  *        alpha, beta and the output type. 0: never (callers that must not allocate). 2..16: that many slices
  *        whenever legal.
+ * key 8: schedule of the straight-line kernel. 0 (default): one workgroup barrier per two k-steps, all loads of a
+ *        loop body behind it (two k-steps to land); 1: a barrier in every k-step, loads spread over both (three
+ *        k-steps to land) - faster when the clock is not power-limited, slower on random operand values.
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

@@ -373,16 +373,19 @@ class StreamModel:
     ahead, in the odd one the two Bt pairs; each pair is two loads (the halves of a line) into quarters
     (j + 4) % 5 and j % 5 of the even k-step j. The odd k-step waits with immediate 4 (+ 32 behind an
     epilogue without C reads); every k-step has one barrier, behind it the fragments of the next k-step
-    are read. Checked: a read finds every wave's share of the expected k-step in the quarter (nothing
+    are read. In the other schedule (odd_only) the even k-step has neither barrier nor loads, the odd one
+    issues all four pairs and waits with immediate 0 (+ 32). Checked: a read finds every wave's share of the expected k-step in the quarter (nothing
     late, nothing overwritten early), and all waves finish."""
 
     LOADS_PER_KSTEP = 4
     STORES = 32
 
-    def __init__(self, waves, bodies_per_item, items, rng, imm=4, imm_stores=36, count_stores=True, completion_rate=0.35, slow_wave=None):
+    def __init__(self, waves, bodies_per_item, items, rng, imm=4, imm_stores=36, count_stores=True, completion_rate=0.35, slow_wave=None,
+                 odd_only=False):
         self.n, self.nb, self.items, self.rng = waves, bodies_per_item, items, rng
         self.completion_rate = completion_rate                       # how eagerly the memory system answers
         self.slow_wave = slow_wave                                   # a wave whose operations complete 50 times more rarely
+        self.odd_only = odd_only                                     # no barrier and no loads in the even k-step (immediates 0 / 32)
         self.imm, self.imm_stores, self.count_stores = imm, imm_stores, count_stores
         self.total = 2 * bodies_per_item * items                     # k-steps in the stream
         # per quarter and wave, per load of a k-step (A rows 16w.., A rows 16(w+8).., Bt likewise): k-step it holds
@@ -436,10 +439,12 @@ class StreamModel:
         stores_in_flight = False
         for j in range(0, self.total, 2):
             # even k-step j
-            yield from barrier()
+            if not self.odd_only:
+                yield from barrier()
             yield
             self.read((j + 1) % 5, j + 1)
-            self.issue_pairs(w, 0, j, j + 4)
+            if not self.odd_only:
+                self.issue_pairs(w, 0, j, j + 4)
             yield
             # odd k-step j + 1
             yield from wait(self.imm_stores if stores_in_flight else self.imm)
@@ -447,6 +452,8 @@ class StreamModel:
             yield
             if j + 2 < self.total:
                 self.read((j + 2) % 5, j + 2)
+            if self.odd_only:
+                self.issue_pairs(w, 0, j, j + 4)
             self.issue_pairs(w, 1, j, j + 4)
             stores_in_flight = False
             if (j + 2) % (2 * self.nb) == 0:                          # the item ends: epilogue
@@ -474,14 +481,20 @@ class StreamModel:
         return None
 
 
+# the two schedules of the kernel: a barrier in every k-step (immediates 4 / 36), or in the odd k-step only (0 / 32)
+SCHEDULES = {"barrier_every_kstep": dict(imm=4, imm_stores=36, odd_only=False), "odd_only": dict(imm=0, imm_stores=32, odd_only=True)}
+
+
+@pytest.mark.parametrize("schedule", sorted(SCHEDULES))
 @pytest.mark.parametrize("bodies,items", [(1, 1), (1, 5), (2, 3), (3, 2), (7, 2), (16, 1)])
-def test_stream_schedule(bodies, items):
+def test_stream_schedule(bodies, items, schedule):
+    kw = SCHEDULES[schedule]
     for seed, rate, slow in ((0, 0.35, None), (1, 0.35, 3), (2, 0.05, None), (3, 0.05, 6)):   # eager, sluggish, one starved wave
-        m = StreamModel(8, bodies, items, random.Random(1000 * bodies + 10 * items + seed), completion_rate=rate, slow_wave=slow)
+        m = StreamModel(8, bodies, items, random.Random(1000 * bodies + 10 * items + seed), completion_rate=rate, slow_wave=slow, **kw)
         assert m.run() is None
         assert not m.errors, m.errors[:3]
     # with C reads in the epilogue the kernel does not count the stores: the stricter immediate is also safe
-    m = StreamModel(8, bodies, items, random.Random(7), count_stores=False)
+    m = StreamModel(8, bodies, items, random.Random(7), count_stores=False, **kw)
     assert m.run() is None and not m.errors
 
 
@@ -499,3 +512,10 @@ def test_stream_model_detects_wrong_immediates():
         m.run()
         caught += bool(m.errors)
     assert caught > 0
+    for imm, imm_stores in ((1, 33), (0, 33)):
+        caught = 0
+        for seed in range(20):
+            m = StreamModel(8, 2, 4, random.Random(seed), imm=imm, imm_stores=imm_stores, completion_rate=0.3, slow_wave=seed % 8, odd_only=True)
+            m.run()
+            caught += bool(m.errors)
+        assert caught > 0
