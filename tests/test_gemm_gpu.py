@@ -594,3 +594,35 @@ def test_split_k_against_the_oracle_and_the_single_pass(ck, oracle):
             ck.set_option(ck.OPT_SPLIT_K, prev)
         assert_close(oracle, ref, out[slices])
     assert_close(oracle, out[0], out[4], rtol=1e-4)
+
+
+def test_straight_line_kernel_random_shapes(ck):
+    # seeded sweep over shapes, grid sizes, tile orders, schedules, epilogue forms and split-K: exact on
+    # small integers whatever the summation order (D starts out as NaN: every element must be written).
+    rng = np.random.default_rng(20240607)
+    for case in range(24):
+        M = int(rng.integers(1, 1100))
+        N = int(rng.integers(1, 1100))
+        K = 64 * int(rng.integers(1, 20))
+        if case % 6 == 5:  # a shape split-K accepts: a multiple of 32 whole-or-ragged tiles, deep K
+            M, N, K = 2048 - int(rng.integers(0, 200)), 1024 - int(rng.integers(0, 50)) * 4, 1024 * int(rng.integers(2, 5))
+        cus = int(rng.choice([1, 2, 3, 5, 8, 64, 256]))
+        group = int(rng.integers(1, 7))
+        dt = ck.DT_F16 if case % 2 == 0 else ck.DT_BF16
+        beta = float(rng.choice([0.0, 0.0, -1.0, 2.0]))
+        every_kstep = int(rng.integers(0, 2))
+        slices = int(rng.choice([0, 1, 2, 4]))
+        t = _straight_line_tuning(ck, cus, group)
+        a = ck.fill_int(dt, (M, K), 97 + case, 0, -2, 2)
+        bt = ck.fill_int(dt, (N, K), 97 + case, 1, -2, 2)
+        c = ck.fill_int(ck.DT_F32, (M, N), 97 + case, 2, -3, 3) if beta else None
+        want = 2.0 * (G.as_f64(dt == ck.DT_BF16, a) @ G.as_f64(dt == ck.DT_BF16, bt).T)
+        if beta:
+            want = want + beta * c.astype(np.float64)
+        prev = (ck.set_option(ck.OPT_BARRIER_EVERY_KSTEP, every_kstep), ck.set_option(ck.OPT_SPLIT_K, slices))
+        try:
+            got = G.run_gemm(ck, dt, a, bt, c, 2.0, beta, t=t)
+        finally:
+            ck.set_option(ck.OPT_BARRIER_EVERY_KSTEP, prev[0])
+            ck.set_option(ck.OPT_SPLIT_K, prev[1])
+        assert np.array_equal(got, want.astype(np.float32)), (case, M, N, K, cus, group, dt, beta, every_kstep, slices)
