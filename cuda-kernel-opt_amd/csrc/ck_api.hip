@@ -174,15 +174,16 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
     a.split_k = 1;
+    a.split_chunk = 32;
     if (g_straight_line.load() &&
         gemm_stream_applies(a, t.tile_dim, t.segment_dim_k, t.num_stages, t.num_producer_waves, t.num_consumer_waves)) {
         // Few tiles and a deep K (fewer tiles than half the CUs): cut K into slices so that every CU has
         // an item, partial products into a stream-ordered workspace, one reduction pass. Needs whole
-        // XCD rounds of tiles (a multiple of 32) and slices of whole loop bodies.
+        // XCD rounds of tiles (a multiple of 32, or fewer than 32) and slices of whole loop bodies.
         int slices = 1;
         const bool bek = g_barrier_every_kstep.load() != 0;
         const int want = g_split_k.load();
-        if (want != 0 && tiles % 32 == 0 && N % 4 == 0) {
+        if (want != 0 && (tiles % 32 == 0 || tiles < 32) && N % 4 == 0) {
             int cand = want >= 2 ? want : (int)(t.num_cus / tiles);
             if (cand > 16) cand = 16;
             while (cand >= 2 && !(K % (cand * STREAM_K_MULTIPLE_HOST) == 0 && K / cand >= 1024)) --cand;
@@ -196,6 +197,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             if (hipMallocAsync((void**)&ws, (size_t)slices * count * sizeof(float), s) != hipSuccess || !ws) return CK_ERR_HIP;
             GemmArgs p = a;
             p.split_k = slices;
+            p.split_chunk = tiles < 32 ? (int)tiles : 32;
             p.D = ws; p.C = nullptr; p.alpha = 1.f; p.beta = 0.f; p.out16 = 0; p.vec_store = 1;
             const int64_t items = tiles * slices;
             const int pgrid = (int)(items < t.num_cus ? items : t.num_cus);

@@ -65,6 +65,7 @@ struct GemmArgs {
     int out16;      // C and D hold the operands' 16-bit element type instead of fp32 (accumulation stays fp32)
     int split_k;    // straight-line kernel only: K is cut into this many slices (>= 1), one work item per (tile, slice);
                     // slice s writes its partial products to D + s * M * N (a workspace; alpha 1, beta 0, fp32)
+    int split_chunk;  // consecutive work items that belong to one slice (32 = one XCD round, or all tiles if fewer)
     uint32_t spin_limit;
     int prio_mode;      // 0: producers at raised priority; 1: also asymmetric consumer burst priorities per SIMD pair; 2: none
     int producer_nap;   // s_sleep argument class of the producers' flag polling: 0 -> 1, 1 -> 4, 2 -> 16

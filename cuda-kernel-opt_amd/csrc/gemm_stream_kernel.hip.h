@@ -82,19 +82,20 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     const int grid = gridDim.x;
     const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
     // Work items: one per (tile, K slice). Item numbers are dealt like tile counts (slot, slot + grid, ...);
-    // 32 consecutive items - what one XCD runs at a time - are 32 consecutive tile counts of ONE slice, so
-    // they share operand panels in that XCD's L2 exactly as whole tiles do. Without split-K an item is
-    // a tile count.
+    // 32 consecutive items - what one XCD runs at a time - are 32 consecutive tile counts of ONE slice
+    // (all tiles, if there are fewer than 32), so they share operand panels in that XCD's L2 exactly as
+    // whole tiles do. Without split-K an item is a tile count.
     const int S = g.split_k;
     const int total_items = g.tiles_m * g.tiles_n * S;
     const int my_tiles = slot < total_items ? (total_items - slot + grid - 1) / grid : 0;
     const int kslice = g.K / S;                  // the host makes this a multiple of one loop body
     const uint32_t kslice_bytes = (uint32_t)kslice * 2u;
     const int nb = kslice / STREAM_K_MULTIPLE;   // loop bodies per item
+    const int CH = g.split_chunk;
     auto item_tile = [&](int64_t item, int& slice) __attribute__((always_inline)) {
-        const int64_t chunk = item / 32;
+        const int64_t chunk = item / CH;
         slice = (int)(chunk % S);
-        return (chunk / S) * 32 + item % 32;
+        return (chunk / S) * CH + item % CH;
     };
 
     // ---- loader ------------------------------------------------------------------------------------

@@ -562,6 +562,8 @@ def test_straight_line_kernel_headline_size_properties(ck):
     (2048, 1024, 8192, 8, 256, "bf16"),
     (2048, 2048, 4096, 1, 256, "f16"),    # automatic: 64 tiles on 256 CUs
     (2000, 1020, 4096, 4, 256, "f16"),    # ragged tiles
+    (512, 768, 8192, 1, 256, "f16"),      # 6 tiles: fewer than one XCD round, automatic slicing (8 slices)
+    (700, 300, 4096, 3, 4, "bf16"),       # 6 ragged tiles on 4 workgroups; 3 slices asked, 4096 has no 3 whole ones: 2
 ])
 def test_split_k_bit_exact(ck, M, N, K, slices, cus, dt_name):
     dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16
