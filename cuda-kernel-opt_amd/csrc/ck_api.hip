@@ -40,7 +40,7 @@ std::atomic<int> g_producer_nap{0};
 std::atomic<int> g_tile_sync_barrier{0};
 std::atomic<int> g_straight_line{1};
 std::atomic<int> g_split_k{1};
-std::atomic<int> g_barrier_every_kstep{0};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
+std::atomic<int> g_barrier_every_kstep{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
 
 constexpr int MAX_DEV = 64;
 std::mutex g_status_mutex;

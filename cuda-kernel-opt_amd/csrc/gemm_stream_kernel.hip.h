@@ -21,11 +21,12 @@
 //     fragments in registers; own loads of k-steps j+2, j+3 landed (the four just issued may fly);
 //     first column; barrier -> quarters q+2, q+3 complete; 7 columns, fragments of j+2 from q+2 and
 //     the four loads of Bt for k-steps j+4 and j+5
-// ODD_ONLY (the default) drops the even k-step's barrier: all four pairs of a body are then issued in the
-// odd k-step, behind its barrier (by then quarter q is free as well), and the odd k-step waits for
-// all of the wave's loads. That leaves the loads two k-steps instead of three and bunches them, which
-// costs 3 % when the clock is fixed (all-zero operands) - and gains 1-1.5 % on random operands, where
-// the device is power-limited and fewer synchronisation points let it hold a higher clock.
+// ODD_ONLY (an option, not the default) drops the even k-step's barrier: all four pairs of a body are
+// then issued in the odd k-step, behind its barrier (by then quarter q is free as well), and the odd
+// k-step waits for all of the wave's loads. That leaves the loads two k-steps instead of three and
+// bunches them: 1.5 % faster at 8192^3 on random operands (the device is power-limited there and holds
+// a higher clock with fewer synchronisation points), but slower wherever the loads take longer
+// (16384^3: 7 %, split-K items: 12 %) or the clock is fixed (all-zero operands: 3 %).
 // The stream of k-steps runs across the tiles of the persistent workgroup; the loader moves to the
 // next tile two bodies before the multiplier does, so its first quarters are in flight while the
 // current tile is finished and written out.

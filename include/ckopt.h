@@ -156,9 +156,10 @@ int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, do
  *        (hipMallocAsync, slices * M * N * 4 bytes) and a second kernel adds them in slice order and applies
  *        alpha, beta and the output type. 0: never (callers that must not allocate). 2..16: that many slices
  *        whenever legal.
- * key 8: schedule of the straight-line kernel. 0 (default): one workgroup barrier per two k-steps, all loads of a
- *        loop body behind it (two k-steps to land); 1: a barrier in every k-step, loads spread over both (three
- *        k-steps to land) - faster when the clock is not power-limited, slower on random operand values.
+ * key 8: schedule of the straight-line kernel. 1 (default): a workgroup barrier in every k-step, the loads of a loop
+ *        body spread over both (three k-steps to land); 0: one barrier per two k-steps, all loads behind it (two
+ *        k-steps to land) - 1.5 % faster at 8192^3 on random operand values (power-limited clock), slower wherever
+ *        memory latency is higher (16384^3: 7 %, split-K: 12 %) or the clock is not power-limited (3 %).
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

@@ -508,7 +508,7 @@ def test_straight_line_kernel_bit_exact(ck, M, N, K, cus, group):
         a = ck.fill_int(dt, (M, K), 91, 0, -2, 2)
         bt = ck.fill_int(dt, (N, K), 91, 1, -2, 2)
         want = (G.as_f64(dt == ck.DT_BF16, a) @ G.as_f64(dt == ck.DT_BF16, bt).T).astype(np.float32)
-        for every_kstep in (0, 1):   # both schedules: barrier in the odd k-step only (default) / in every k-step
+        for every_kstep in (0, 1):   # both schedules: barrier in the odd k-step only / in every k-step (default)
             prev = ck.set_option(ck.OPT_BARRIER_EVERY_KSTEP, every_kstep)
             try:
                 got = G.run_gemm(ck, dt, a, bt, t=t)
