@@ -114,11 +114,8 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
     if (!g.out16) {
         if (interior) {
             if (beta != 0.f) v += *(const f32x4*)(g.C + off) * beta;
-#if defined(CK_NT_STORE)  // D is written once and not read again: keep it from displacing the operands in L2
+            // D is written once and not read again: non-temporal, so that it does not displace the operands in L2
             __builtin_nontemporal_store(v, (f32x4*)(g.D + off));
-#else
-            *(f32x4*)(g.D + off) = v;
-#endif
         } else if (m < g.M) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -143,12 +140,8 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
             uint2 o;
             o.x = (uint32_t)Out16<DT>::store(v[0]) | ((uint32_t)Out16<DT>::store(v[1]) << 16);
             o.y = (uint32_t)Out16<DT>::store(v[2]) | ((uint32_t)Out16<DT>::store(v[3]) << 16);
-#if defined(CK_NT_STORE)
             typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
             __builtin_nontemporal_store(u32x2{o.x, o.y}, (u32x2*)(d16 + off));
-#else
-            *(uint2*)(d16 + off) = o;
-#endif
         } else if (m < g.M) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {

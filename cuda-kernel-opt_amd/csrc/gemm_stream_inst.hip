@@ -1,5 +1,4 @@
 // Launchers of the straight-line 256 x 256 kernel (one instance per element type).
-#define CK_NT_STORE 1
 #include "gemm_stream_kernel.hip.h"
 
 namespace ck {
