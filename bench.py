@@ -144,7 +144,12 @@ def main():
     cus = args.cus or torch.cuda.get_device_properties(0).multi_processor_count
 
     kind, dtype, M, N, K, dist = WORKLOADS[args.workload]
-    tuned = TUNED.get(args.workload, (256, 64, 2, 2, 8))
+    # tuning flags default to what the library suggests for the shape (ckopt_suggest_gemm_tuning); TUNED records
+    # what that is for the named workloads and is checked against it
+    sug = ck.suggest_gemm_tuning(M, N, K, cus)
+    tuned = (sug["tile_dim"], sug["segment_dim_k"], sug["num_stages"], sug["num_producer_warps"], sug["num_consumer_warps"])
+    if kind == "gemm" and args.workload in TUNED and tuned != TUNED[args.workload]:
+        print("note: suggestion %s differs from the recorded tuple %s" % (tuned, TUNED[args.workload]), file=sys.stderr)
     for name, val in zip(("tile", "segk", "stages", "producers", "consumers"), tuned):
         if getattr(args, name) is None:
             setattr(args, name, val)

@@ -58,6 +58,8 @@ _lib.ckopt_probe_counters.restype = _i
 _lib.ckopt_probe_counters.argtypes = [_p, ctypes.POINTER(ctypes.c_uint), _i]
 _lib.ckopt_probe_mfma_ceiling.restype = _i
 _lib.ckopt_probe_mfma_ceiling.argtypes = [_i, _i, _i, ctypes.POINTER(ctypes.c_double)]
+_lib.ckopt_suggest_gemm_tuning.restype = _i
+_lib.ckopt_suggest_gemm_tuning.argtypes = [_i, _i, _i, _i, ctypes.POINTER(ctypes.c_int)]
 _lib.ckopt_set_option.restype = _i
 _lib.ckopt_set_option.argtypes = [_i, _i]
 _lib.ckopt_fill_uniform.restype = _i
@@ -76,6 +78,7 @@ EXPORTED_SYMBOLS = [
     "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
     "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks", "ckopt_probe_counters",
+    "ckopt_suggest_gemm_tuning",
     "ckopt_probe_mfma_ceiling",
     "ckopt_set_option", "ckopt_fill_uniform",
     "ckopt_fill_normal", "ckopt_fill_int", "ckopt_fill_constant", "ckopt_error_string",
@@ -234,6 +237,17 @@ def probe_counters(nwaves=16, stream=None):
     buf = (ctypes.c_uint * (nwaves * 8))()
     _check(_lib.ckopt_probe_counters(_stream(stream), buf, nwaves * 8), "probe_counters")
     return [list(buf[w * 8:(w + 1) * 8]) for w in range(nwaves)]
+
+
+def suggest_gemm_tuning(M, N, K, num_cus=256):
+    """Tuning tuple for a problem size: dict with the launcher's parameter names."""
+    out = (ctypes.c_int * 10)()
+    _check(_lib.ckopt_suggest_gemm_tuning(M, N, K, num_cus, out), "suggest_gemm_tuning")
+    names = ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
+             "num_stages", "num_producer_warps", "num_consumer_warps")
+    d = dict(zip(names, [int(v) for v in out]))
+    d["num_sms"] = num_cus
+    return d
 
 
 def set_option(key, value):

@@ -40,7 +40,8 @@ std::atomic<int> g_producer_nap{0};
 std::atomic<int> g_tile_sync_barrier{0};
 std::atomic<int> g_straight_line{1};
 std::atomic<int> g_split_k{1};
-std::atomic<int> g_barrier_every_kstep{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
+std::atomic<int> g_barrier_every_kstep{1};
+constexpr int SPLIT_K_MIN_SLICE = 1024;  // shortest K slice split-K will make (shorter ones lose more in the reduction pass than they gain)  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
 
 constexpr int MAX_DEV = 64;
 std::mutex g_status_mutex;
@@ -186,7 +187,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         if (want != 0 && (tiles % 32 == 0 || tiles < 32) && N % 4 == 0) {
             int cand = want >= 2 ? want : (int)(t.num_cus / tiles);
             if (cand > 16) cand = 16;
-            while (cand >= 2 && !(K % (cand * STREAM_K_MULTIPLE_HOST) == 0 && K / cand >= 1024)) --cand;
+            while (cand >= 2 && !(K % (cand * STREAM_K_MULTIPLE_HOST) == 0 && K / cand >= SPLIT_K_MIN_SLICE)) --cand;
             if (cand >= 2 && (want >= 2 || tiles * 2 <= t.num_cus)) slices = cand;
         }
         if (slices == 1) {
@@ -317,6 +318,33 @@ int ckopt_check_gemm_tuning(int tile_dim, int segment_dim_k, int bar_steps_a, in
     const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
                            tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
     return ck::check_gemm_tuning(t);
+}
+
+int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out) {
+    using namespace ck;
+    if (!tuning_out) return CK_ERR_NULL;
+    if (M <= 0 || N <= 0 || K <= 0 || num_cus <= 0) return CK_ERR_BAD_PARAM;
+    auto tiles = [&](int t) { return (int64_t)((M + t - 1) / t) * ((N + t - 1) / t); };
+    const int kp = (K + CHUNK_ELEMS - 1) / CHUNK_ELEMS * CHUNK_ELEMS;  // what the kernels see after the repack
+    // {tile, seg_k, bar_steps_a, bar_steps_b, rows_a, rows_b, group, stages, producers, consumers}
+    static const int straight_line[10] = {256, 32, 0, 0, 256, 256, 4, 5, 0, 8};
+    static const int fused_128[10] = {128, 128, 0, 0, 128, 128, 4, 2, 0, 8};
+    static const int fused_64[10] = {64, 128, 0, 0, 64, 64, 4, 4, 0, 8};
+    static const int pc_256[10] = {256, 64, 0, 0, 256, 256, 4, 2, 2, 8};
+    const int* pick = fused_64;
+    const int64_t t256 = tiles(256);
+    bool split_ok = false;
+    if (kp % STREAM_K_MULTIPLE_HOST == 0 && (t256 % 32 == 0 || t256 < 32) && N % 4 == 0 && t256 * 2 <= num_cus) {
+        int cand = (int)(num_cus / t256);
+        if (cand > 16) cand = 16;
+        while (cand >= 2 && !(kp % (cand * STREAM_K_MULTIPLE_HOST) == 0 && kp / cand >= SPLIT_K_MIN_SLICE)) --cand;
+        split_ok = cand >= 4;  // two slices gain less than the reduction pass costs
+    }
+    if (t256 * 2 >= num_cus) pick = kp % STREAM_K_MULTIPLE_HOST == 0 ? straight_line : pc_256;
+    else if (split_ok) pick = straight_line;
+    else if (tiles(128) * 2 >= num_cus) pick = fused_128;
+    for (int i = 0; i < 10; ++i) tuning_out[i] = pick[i];
+    return CK_OK;
 }
 
 int ckopt_matmul_shmem(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int tile_dim,

@@ -98,6 +98,14 @@ int ckopt_check_gemm_tuning(int tile_dim, int segment_dim_k, int bar_steps_a, in
                             int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
                             int num_producer_waves, int num_consumer_waves, int num_cus);
 
+/* A tuning tuple for a problem size, from the measurements on MI355X (no counterpart in the reference, whose
+ * drivers sweep the tuples by hand, port_2.cu:1463-1480): tuning_out receives {tile_dim, segment_dim_k,
+ * bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+ * num_consumer_warps} in the launcher's parameter order. Enough 256 x 256 tiles for half the CUs (or a K deep
+ * enough to be cut into at least four slices): the straight-line kernel's tuple; else 128 x 128 tiles if those
+ * occupy half the CUs; else 64 x 64 tiles. */
+int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out);
+
 /* Replaces matmul_shmem<DT,DT_ACC>() of matmul_shmem.cu:143-174: C = A * B without matrix cores.
  * dtype CKOPT_DT_F32 (fp32 in, fp32 accumulate), CKOPT_DT_F16 (fp16 in/out, fp32 accumulate) or
  * CKOPT_DT_I32 (exact). A: M x K, C: M x N row-major. b_transposed == 0: B is K x N row-major as in

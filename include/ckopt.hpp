@@ -102,6 +102,18 @@ int get_shmem_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_step
     if (r < 0) throw Error(r, "get_shmem_req");
     return r;
 }
+// tuning tuple for a problem size in the launcher's parameter order (no counterpart in the reference)
+struct Tuning {
+    int tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages,
+        num_producer_warps, num_consumer_warps;
+};
+inline Tuning suggest_gemm_tuning(int M, int N, int K, int num_sms) {
+    int v[10];
+    const int r = ckopt_suggest_gemm_tuning(M, N, K, num_sms, v);
+    if (r < 0) throw Error(r, "suggest_gemm_tuning");
+    return Tuning{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9]};
+}
+
 inline int get_num_acc(int tile_dim, int num_consumer_warps) {
     const int r = ckopt_get_num_acc(tile_dim, num_consumer_warps);
     if (r < 0) throw Error(r, "get_num_acc");

@@ -204,3 +204,27 @@ def test_option_keys_reject_values_outside_their_range(ck):
     assert ck.set_option(ck.OPT_SPLIT_K, prev) == 0
     prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
     assert ck.set_option(ck.OPT_STRAIGHT_LINE, prev) == 0
+
+
+def test_suggested_tunings_are_legal_and_follow_the_measured_rules(ck):
+    # every suggestion passes the launcher's own validation; the BASELINE shapes get the tuples bench.py uses
+    import itertools
+    for M, N, K in itertools.product((1, 100, 512, 1024, 2048, 3000, 8192), (4, 130, 1024, 4097), (8, 64, 1000, 3071, 32768)):
+        t = ck.suggest_gemm_tuning(M, N, K)
+        assert ck.check_gemm_tuning(t["tile_dim"], t["segment_dim_k"], t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"],
+                                    t["bar_step_rows_b"], t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                    t["num_consumer_warps"], t["num_sms"]) == 0, (M, N, K, t)
+    straight = dict(tile_dim=256, segment_dim_k=32, num_stages=5, num_producer_warps=0, num_consumer_warps=8)
+    def picks(M, N, K):
+        t = ck.suggest_gemm_tuning(M, N, K)
+        return {k: t[k] for k in straight}
+    assert picks(8192, 8192, 8192) == straight          # config 3
+    assert picks(2048, 2048, 32768) == straight         # config 4: 64 tiles, four slices of 8192
+    assert picks(6143, 4097, 3071) == straight          # config 5: K is 3072 after the repack
+    assert picks(16384, 16384, 16384) == straight
+    assert picks(1024, 1024, 8192) == straight          # 16 tiles, eight slices of 1024
+    assert picks(2048, 2048, 2048)["tile_dim"] == 128   # 64 tiles of 256 and K too shallow to cut four times
+    assert picks(512, 512, 512)["tile_dim"] == 64       # config 1
+    assert picks(8192, 8192, 8200)["num_producer_warps"] == 2 and picks(8192, 8192, 8200)["tile_dim"] == 256  # K % 64 != 0
+    with pytest.raises(ck.CkoptError):
+        ck.suggest_gemm_tuning(0, 1, 1)
