@@ -69,14 +69,31 @@ __global__ void pad_rows_kernel(const unsigned short* __restrict__ src, unsigned
     const long long total = (long long)rows * chunks_per_row;
     for (long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x; c < total; c += (long long)gridDim.x * blockDim.x) {
         const int r = (int)(c / chunks_per_row), k0 = (int)(c % chunks_per_row) * 8;
-        const unsigned short* s = src + (long long)r * K + k0;
-        unsigned short v[8];
+        // The chunk's 16 source bytes start on a 2-byte boundary: five aligned 4-byte words cover them,
+        // shifted by two bytes where the start is odd. A word that lies only half inside
+        // [chunk start, row end) is read as that one element, so no byte outside the row is touched.
+        const uintptr_t first = (uintptr_t)(src + (long long)r * K + k0);
+        const uintptr_t row_end = (uintptr_t)(src + (long long)r * K + K);
+        const uintptr_t w0 = first & ~(uintptr_t)3;
+        const bool odd = (first & 2) != 0;
+        unsigned d[5];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = k0 + e < K ? s[e] : (unsigned short)0;
-        uint4 o;
-        o.x = v[0] | ((unsigned)v[1] << 16); o.y = v[2] | ((unsigned)v[3] << 16);
-        o.z = v[4] | ((unsigned)v[5] << 16); o.w = v[6] | ((unsigned)v[7] << 16);
-        *reinterpret_cast<uint4*>(dst + (long long)r * Kp + k0) = o;
+        for (int i = 0; i < 5; ++i) {
+            const uintptr_t lo = w0 + 4 * i, hi = lo + 2;
+            const bool lo_in = lo >= first && lo < row_end, hi_in = hi >= first && hi < row_end;
+            if (lo_in && hi_in) d[i] = *reinterpret_cast<const unsigned*>(lo);
+            else d[i] = (lo_in ? (unsigned)*reinterpret_cast<const unsigned short*>(lo) : 0u) |
+                        (hi_in ? (unsigned)*reinterpret_cast<const unsigned short*>(hi) << 16 : 0u);
+        }
+        unsigned o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[i] = odd ? (d[i] >> 16) | (d[i + 1] << 16) : d[i];
+            const int k = k0 + 2 * i;  // elements k, k + 1 of the row: zero where the row has ended
+            if (k >= K) o[i] = 0u;
+            else if (k + 1 >= K) o[i] &= 0xffffu;
+        }
+        *reinterpret_cast<uint4*>(dst + (long long)r * Kp + k0) = uint4{o[0], o[1], o[2], o[3]};
     }
 }
 
