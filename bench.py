@@ -78,6 +78,62 @@ def cpu_baseline(ck, kind, dtype, a, b, M, N, K, budget_s=12.0):
                       "matmul_test.h:289-302 vectorised across output columns, %d OpenMP threads" % (rows, M, dt, threads)}
 
 
+def sweep(ck, torch, args, ckdt, da, db, dd, M, N, K, cus, stream):
+    """Times a list of tuning tuples: (tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
+    bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps): TFLOP/s per line, the
+    format of the reference's performance loops, then one JSON line with all of them and the best."""
+    tuples = []
+    for tile, c in ((256, 8), (128, 8), (128, 4), (64, 8), (64, 4)):
+        wtr = ck.get_warp_tile_rows(tile, c)
+        wave_rows = (wtr * 16, ck.get_num_acc(tile, c) // wtr * 16)
+        for segk, stages, p in ((32, 5, 0), (32, 4, 0), (64, 2, 0), (128, 2, 0), (64, 2, 2), (64, 2, 4), (32, 4, 4), (64, 4, 2), (64, 4, 4), (128, 2, 2)):
+            tuples.append((tile, segk, 0, 0, tile, tile, args.group, stages, p, c))
+        if tile >= 128:   # the finer synchronisation granularities of port_1 / port_2 (producer/consumer kernels only)
+            tuples.append((tile, 64, 2, 1, wave_rows[0], wave_rows[1], args.group, 2 if tile == 256 else 4, 2, c))
+            tuples.append((tile, 64, c // 2, 2, wave_rows[0], wave_rows[1], args.group, 2 if tile == 256 else 4, 2, c))
+            tuples.append((tile, 64, 1, 3 if tile == 256 or c == 4 else 1, 16, 16, args.group, 2 if tile == 256 else 4, 2, c))
+    for g in (1, 2, 8):   # tile order: row-major (1) and other group sizes, on the suggested tuple
+        sg = ck.suggest_gemm_tuning(M, N, K, cus)
+        tuples.append((sg["tile_dim"], sg["segment_dim_k"], 0, 0, sg["bar_step_rows_a"], sg["bar_step_rows_b"], g, sg["num_stages"],
+                       sg["num_producer_warps"], sg["num_consumer_warps"]))
+    flops = 2.0 * M * N * K
+    reps = max(args.steps // 10, 5)
+    rows = []
+    warm = tuples[0]   # bring the device to its steady clock before the first tuple is timed
+    for _ in range(max(args.warmup, 1) * 3):
+        ck.gemm_shmem_tc_async_opt_port(ckdt, da, db, None, dd, 1.0, 0.0, M, N, K, *warm, cus, stream)
+    torch.cuda.synchronize()
+    for t in tuples:
+        if ck.check_gemm_tuning(*t, cus) != 0:
+            continue
+        def step():
+            ck.gemm_shmem_tc_async_opt_port(ckdt, da, db, None, dd, 1.0, 0.0, M, N, K, t[0], t[1], t[2], t[3], t[4], t[5], t[6], t[7], t[8],
+                                            t[9], cus, stream)
+        try:
+            for _ in range(3):
+                step()
+        except ck.CkoptError:
+            continue   # no instance for this tuple
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for _ in range(reps):
+            step()
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        if ck.device_status() != 0:
+            print("device status non-zero for %s" % (t,), file=sys.stderr)
+            return 4
+        tf = flops / (ev0.elapsed_time(ev1) / reps * 1e-3) * 1e-12
+        print("(%s): %.2f" % (", ".join(str(v) for v in t), tf), flush=True)
+        rows.append({"tuple": list(t), "tflops": round(tf, 2)})
+    best = max(rows, key=lambda r: r["tflops"])
+    print(json.dumps({"sweep": args.workload, "unit": "TFLOP/s", "reps": reps, "tuple_order": "tile_dim, segment_dim_k, bar_steps_a, "
+                      "bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps",
+                      "results": rows, "best": best}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -106,6 +162,9 @@ def main():
     ap.add_argument("--no-ceiling", action="store_true", help="skip the bare inner-loop probe of the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--sweep", action="store_true",
+                    help="time a list of tuning tuples on the workload (the role of the reference drivers' performance "
+                         "loops, port_2.cu:1463-1480): one line per tuple in the reference's format, then one JSON line")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -169,6 +228,8 @@ def main():
     dd = torch.empty((M, N), dtype=torch.float32, device=dev)
     stream = torch.cuda.current_stream()
 
+    if kind == "gemm" and args.sweep:
+        return sweep(ck, torch, args, ckdt, da, db, dd, M, N, K, cus, stream)
     if kind == "gemm":
         rows_a = rows_b = args.tile
         if args.mode == "wave":
