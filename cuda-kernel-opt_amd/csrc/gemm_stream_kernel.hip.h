@@ -247,6 +247,10 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         }
     };
 
+    // The two waves of a SIMD run the same code in step; at different priorities one leads and the other
+    // fills in while the leader fetches, instead of both fetching and both multiplying at the same moments
+    // (+0.7 % on random operands, nothing on all-zero ones).
+    if (wave & 4) __builtin_amdgcn_s_setprio(3);
     if (my_tiles > 0) {
         // prologue: the first two bodies' quarters, then the fragments of k-step 0
         loader_open_tile();
