@@ -39,9 +39,9 @@ std::atomic<int> g_prio_mode{0};
 std::atomic<int> g_producer_nap{0};
 std::atomic<int> g_tile_sync_barrier{0};
 std::atomic<int> g_straight_line{1};
-std::atomic<int> g_split_k{1};
+std::atomic<int> g_split_k{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
 std::atomic<int> g_barrier_every_kstep{1};
-constexpr int SPLIT_K_MIN_SLICE = 1024;  // shortest K slice split-K will make (shorter ones lose more in the reduction pass than they gain)  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
+constexpr int SPLIT_K_MIN_SLICE = 1024;  // shortest K slice split-K will make (shorter ones lose more in the reduction pass than they gain)
 
 constexpr int MAX_DEV = 64;
 std::mutex g_status_mutex;
@@ -120,6 +120,21 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int slices, l
 int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
                 int N, int K, const ck::GemmTuning& t, void* stream, int out16);
 
+// Number of K slices the straight-line kernel uses for `tiles` 256 x 256 tiles (1: no split). policy 0: never;
+// 1: automatic - fewer tiles than half the CUs and at least four legal slices (two gain less than the
+// reduction pass costs); >= 2: that many slices if legal, else the next smaller legal count. Legal: whole XCD
+// rounds of tiles (a multiple of 32, or fewer than 32), N % 4 == 0 (vector stores of the partial planes), slices
+// of whole loop bodies and at least SPLIT_K_MIN_SLICE deep.
+int split_k_slices(int64_t tiles, int N, int K, int num_cus, int policy) {
+    if (policy == 0 || !(tiles % 32 == 0 || tiles < 32) || N % 4 != 0) return 1;
+    int cand = policy >= 2 ? policy : (int)(num_cus / tiles);
+    if (cand > 16) cand = 16;
+    while (cand >= 2 && !(K % (cand * ck::STREAM_K_MULTIPLE_HOST) == 0 && K / cand >= SPLIT_K_MIN_SLICE)) --cand;
+    if (cand < 2) return 1;
+    if (policy >= 2) return cand;
+    return tiles * 2 <= num_cus && cand >= 4 ? cand : 1;
+}
+
 // K % 8 != 0 or operands off a 16-byte boundary: the product is computed from zero-padded,
 // aligned copies of A and Bt in a stream-ordered temporary (zeros in the K tail add nothing).
 int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta,
@@ -195,18 +210,10 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     a.split_chunk = 32;
     if (g_straight_line.load() &&
         gemm_stream_applies(a, t.tile_dim, t.segment_dim_k, t.num_stages, t.num_producer_waves, t.num_consumer_waves)) {
-        // Few tiles and a deep K (fewer tiles than half the CUs): cut K into slices so that every CU has
-        // an item, partial products into a stream-ordered workspace, one reduction pass. Needs whole
-        // XCD rounds of tiles (a multiple of 32, or fewer than 32) and slices of whole loop bodies.
-        int slices = 1;
+        // Few tiles and a deep K: cut K into slices so that every CU has an item, partial products into
+        // a stream-ordered workspace, one reduction pass.
         const bool bek = g_barrier_every_kstep.load() != 0;
-        const int want = g_split_k.load();
-        if (want != 0 && (tiles % 32 == 0 || tiles < 32) && N % 4 == 0) {
-            int cand = want >= 2 ? want : (int)(t.num_cus / tiles);
-            if (cand > 16) cand = 16;
-            while (cand >= 2 && !(K % (cand * STREAM_K_MULTIPLE_HOST) == 0 && K / cand >= SPLIT_K_MIN_SLICE)) --cand;
-            if (cand >= 2 && (want >= 2 || tiles * 2 <= t.num_cus)) slices = cand;
-        }
+        const int slices = split_k_slices(tiles, N, K, t.num_cus, g_split_k.load());
         if (slices == 1) {
             e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a, bek) : launch_gemm_stream_bf16(dim3(grid), s, a, bek);
         } else {
@@ -350,13 +357,7 @@ int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out)
     static const int pc_256[10] = {256, 64, 0, 0, 256, 256, 4, 2, 2, 8};
     const int* pick = fused_64;
     const int64_t t256 = tiles(256);
-    bool split_ok = false;
-    if (kp % STREAM_K_MULTIPLE_HOST == 0 && (t256 % 32 == 0 || t256 < 32) && N % 4 == 0 && t256 * 2 <= num_cus) {
-        int cand = (int)(num_cus / t256);
-        if (cand > 16) cand = 16;
-        while (cand >= 2 && !(kp % (cand * STREAM_K_MULTIPLE_HOST) == 0 && kp / cand >= SPLIT_K_MIN_SLICE)) --cand;
-        split_ok = cand >= 4;  // two slices gain less than the reduction pass costs
-    }
+    const bool split_ok = kp % STREAM_K_MULTIPLE_HOST == 0 && split_k_slices(t256, N, kp, num_cus, 1) > 1;
     if (t256 * 2 >= num_cus) pick = kp % STREAM_K_MULTIPLE_HOST == 0 ? straight_line : pc_256;
     else if (split_ok) pick = straight_line;
     else if (tiles(128) * 2 >= num_cus) pick = fused_128;

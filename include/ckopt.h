@@ -159,8 +159,8 @@ int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, do
  *        tiles (M, N multiples of 256) and K a multiple of 64 take the straight-line kernel written for exactly
  *        that shape (gemm_stream_kernel; default 1); 0 sends them through the general fused kernel.
  * key 7: split-K of the straight-line kernel. 1 (default): when a launch has fewer tiles than half the CUs (a
- *        multiple of 32 of them, or fewer than 32; N % 4 == 0, slices of at least 1024 that are multiples of 64), K is cut into
- *        num_sms / tiles slices (at most 16); the slices' partial products go to a stream-ordered temporary
+ *        multiple of 32 of them, or fewer than 32; N % 4 == 0) and K allows at least four slices of at least 1024
+ *        that are multiples of 64, K is cut into num_sms / tiles slices (at most 16); the slices' partial products go to a stream-ordered temporary
  *        (hipMallocAsync, slices * M * N * 4 bytes) and a second kernel adds them in slice order and applies
  *        alpha, beta and the output type. 0: never (callers that must not allocate). 2..16: that many slices
  *        whenever legal.
