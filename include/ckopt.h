@@ -155,13 +155,14 @@ int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, do
  *        consumer bursts per SIMD pair, 2 none); key 4: producers' polling nap (0, 1, 2 = s_sleep 1, 4, 16);
  * key 5: tile granularity with dedicated producers synchronises through the hardware workgroup barrier
  *        (gemm_pcb_kernel, needs num_stages >= 2) instead of LDS counters (default 0).
- * key 6: launches with num_producer_warps 0, tile_dim 256, segment_dim_k 32, num_stages 5, 8 consumer warps, whole
- *        tiles (M, N multiples of 256) and K a multiple of 64 take the straight-line kernel written for exactly
- *        that shape (gemm_stream_kernel; default 1); 0 sends them through the general fused kernel.
+ * key 6: launches with num_producer_warps 0, tile_dim 256, segment_dim_k 32, num_stages 5, 8 consumer warps and K a
+ *        multiple of 64 (any M, N) take the straight-line kernel written for exactly that shape
+ *        (gemm_stream_kernel; default 1); 0 sends them through the general fused kernel.
  * key 7: split-K of the straight-line kernel. 1 (default): when a launch has fewer tiles than half the CUs (a
  *        multiple of 32 of them, or fewer than 32; N % 4 == 0) and K allows at least four slices of at least 1024
- *        that are multiples of 64, K is cut into num_sms / tiles slices (at most 16); the slices' partial products go to a stream-ordered temporary
- *        (hipMallocAsync, slices * M * N * 4 bytes) and a second kernel adds them in slice order and applies
+ *        that are multiples of 64, K is cut into num_sms / tiles slices (at most 16); the slices' partial products
+ *        go to a stream-ordered temporary (hipMallocAsync, slices * M * N * 4 bytes) and a second kernel adds
+ *        them in slice order and applies
  *        alpha, beta and the output type. 0: never (callers that must not allocate). 2..16: that many slices
  *        whenever legal.
  * key 8: schedule of the straight-line kernel. 1 (default): a workgroup barrier in every k-step, the loads of a loop
