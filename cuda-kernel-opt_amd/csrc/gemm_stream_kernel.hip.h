@@ -168,13 +168,19 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < WTC; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // 1 when beta is (plus or minus) zero: then the epilogue is 32 stores and nothing else. Worked out on
-    // the scalar unit in asm: a flag the compiler derives from a float compare ends up in a vector
-    // register, which the "s" operands of the asm statements below cannot take.
-    uint32_t count_stores;
-    asm volatile("s_lshl_b32 %0, %1, 1\n\ts_cmp_eq_u32 %0, 0\n\ts_cselect_b32 %0, 1, 0"
-                 : "=&s"(count_stores)
-                 : "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, g.beta)))
+    // How many stores an interior tile's epilogue leaves in flight, as the code the landing wait takes:
+    // 0 = wait for everything (beta is not zero: the epilogue also loads C), 2 = 32 stores (beta is plus or
+    // minus zero), 1 = 16 stores (beta zero, 16-bit output through the 16-byte store path below, which
+    // needs D and its rows on 16-byte boundaries). Worked out on the scalar unit in asm: a flag the compiler
+    // derives from a compare ends up in a vector register, which the "s" operands of the asm statements
+    // below cannot take.
+    const uint32_t d16_misaligned = ((uint32_t)(uintptr_t)g.D | ((uint32_t)g.N << 1)) & 15u;
+    uint32_t count_stores, count_tmp;
+    asm volatile("s_lshl_b32 %0, %2, 1\n\ts_cmp_eq_u32 %0, 0\n\ts_cselect_b32 %0, 2, 0\n\t"
+                 "s_cmp_eq_u32 %4, 0\n\ts_cselect_b32 %1, %3, 0\n\ts_lshr_b32 %0, %0, %1"
+                 : "=&s"(count_stores), "=&s"(count_tmp)
+                 : "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, g.beta))),
+                   "s"(__builtin_amdgcn_readfirstlane((uint32_t)g.out16)), "s"(__builtin_amdgcn_readfirstlane(d16_misaligned))
                  : "scc");
 #if defined(CK_PROBE_TIMING)  // measurement build only: cycles in the epilogues, in the first and second loop body behind one, in all others
     unsigned long long t_epi = 0, t_first = 0, t_second = 0, t_other = 0;
@@ -196,9 +202,11 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             // between the two immediates is a scalar branch inside one asm statement: a branch the
             // compiler can see would split the k-step into basic blocks with all 224 accumulator
             // and fragment registers live across them.)
-            asm volatile("s_cmp_lg_u32 %0, 0\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(%1)\n1:\n\ts_waitcnt vmcnt(%2)"
+            asm volatile("s_cmp_lg_u32 %0, 0\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(%1)\n1:\n\t"
+                         "s_cmp_eq_u32 %0, 2\n\ts_cbranch_scc1 2f\n\ts_waitcnt vmcnt(%2)\n2:\n\ts_waitcnt vmcnt(%3)"
                          :
-                         : "s"(stores_in_flight), "n"(ODD_ONLY ? 0 : LPB / 2), "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES)
+                         : "s"(stores_in_flight), "n"(ODD_ONLY ? 0 : LPB / 2), "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES / 2),
+                           "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES)
                          : "memory", "scc");
         }
 #endif
@@ -339,6 +347,52 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                             const int64_t off = (row0 + i * 16 + tt * 8) * g.N + (col0 + j * 16);
                             if (beta != 0.f) v += *(const f32x4*)(go.C + off) * beta;
                             __builtin_nontemporal_store(v, (f32x4*)(go.D + off));
+                        }
+                    }
+                }
+            } else if (interior && g.out16 && d16_misaligned == 0 && g.beta == 0.f) {
+                // 16-bit output in whole 128-byte lines, 16 bytes per lane. A lane's 4 results of a block are
+                // 8 bytes, so two neighbouring blocks swap their odd and even 16-lane rows
+                // (v_permlane16_swap): lane group G = lane / 16 then holds the 8 columns 8 (G / 2) .. of block
+                // j + G % 2, and the 4 lanes of a row 64 consecutive bytes. Two such pairs make a line: the
+                // lanes of rows 8 .. 15 hand the second pair's piece to rows 0 .. 7 and take theirs (a
+                // rotation by 8 inside each 16-lane row, a DPP move), so that store t writes rows
+                // 8t .. 8t+7, first pair from the lanes that own those rows, second pair from the others.
+                unsigned short* d16 = (unsigned short*)go.D;
+                const bool low_rows = lr < 8;
+                const int unit = ((lg & 1) * 2 + (lg >> 1)) * 8;   // column of the lane's piece inside a pair's 32
+                const int64_t row0 = (int64_t)(rc.row * TILE + R * WTR * 16 + (lr & 7));
+                const int col0 = rc.col * TILE + Cc * WTC * 16 + unit;
+                const float alpha = g.alpha;
+                typedef uint32_t pair_u32 __attribute__((ext_vector_type(2)));
+                auto packed_pair = [&](f32x4 x0, f32x4 x1) __attribute__((always_inline)) {
+                    const f32x4 v0 = x0 * alpha, v1 = x1 * alpha;
+                    const uint32_t p00 = (uint32_t)Out16<DT>::store(v0[0]) | ((uint32_t)Out16<DT>::store(v0[1]) << 16);
+                    const uint32_t p01 = (uint32_t)Out16<DT>::store(v0[2]) | ((uint32_t)Out16<DT>::store(v0[3]) << 16);
+                    const uint32_t p10 = (uint32_t)Out16<DT>::store(v1[0]) | ((uint32_t)Out16<DT>::store(v1[1]) << 16);
+                    const uint32_t p11 = (uint32_t)Out16<DT>::store(v1[2]) | ((uint32_t)Out16<DT>::store(v1[3]) << 16);
+                    const pair_u32 s0 = __builtin_amdgcn_permlane16_swap(p00, p10, false, false);
+                    const pair_u32 s1 = __builtin_amdgcn_permlane16_swap(p01, p11, false, false);
+                    return u32x4{s0[0], s1[0], s0[1], s1[1]};
+                };
+#pragma unroll
+                for (int i = 0; i < WTR; ++i) {
+#pragma unroll
+                    for (int j = 0; j < WTC; j += 4) {
+                        const u32x4 first = packed_pair(acc[i][j], acc[i][j + 1]);
+                        const u32x4 second = packed_pair(acc[i][j + 2], acc[i][j + 3]);
+                        u32x4 other;  // the second pair's piece of the row 8 away
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            other[e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)second[e], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+#pragma unroll
+                        for (int tt = 0; tt < 2; ++tt) {
+                            const bool own = low_rows == (tt == 0);  // this lane's row is among the store's 8 rows
+                            u32x4 o;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) o[e] = own ? first[e] : other[e];
+                            const int64_t off = (row0 + i * 16 + tt * 8) * g.N + (col0 + j * 16 + (own ? 0 : 32));
+                            __builtin_nontemporal_store(o, (u32x4*)(d16 + off));
                         }
                     }
                 }

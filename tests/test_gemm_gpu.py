@@ -540,6 +540,64 @@ def test_straight_line_kernel_epilogue_and_general_kernel_agree(ck, oracle):
     assert_close(oracle, general, got)
 
 
+@pytest.mark.parametrize("dt_name", ["f16", "bf16"])
+@pytest.mark.parametrize("N", [776, 772])   # rows of D on 16-byte boundaries (16 bytes per lane and store) and not
+def test_straight_line_kernel_16_bit_output(ck, oracle, dt_name, N):
+    # the <half, half> role through the straight-line kernel: interior tiles take the 16-byte store path
+    # (two blocks exchanged between lanes), edge tiles and unaligned rows the general one
+    dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16
+    odt = oracle.DT_F16 if dt_name == "f16" else oracle.DT_BF16
+    is_bf = dt_name == "bf16"
+    tdt = torch.bfloat16 if is_bf else torch.float16
+
+    def run(a, bt, c16, alpha, beta, M, K, cus, schedule=1, straight_line=1):
+        t = _straight_line_tuning(ck, cus=cus)
+        da, db = G.to_dev(a), G.to_dev(bt)
+        dc = None if c16 is None else G.to_dev(c16)
+        dd = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+        prev = ck.set_option(ck.OPT_BARRIER_EVERY_KSTEP, schedule), ck.set_option(ck.OPT_STRAIGHT_LINE, straight_line)
+        try:
+            ck.gemm_shmem_tc_async_opt_port_lp(dt, da, db, dc, dd, alpha, beta, M, N, K, t["tile_dim"], t["segment_dim_k"],
+                                               t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                               t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                               t["num_consumer_warps"], t["num_sms"])
+        finally:
+            ck.set_option(ck.OPT_BARRIER_EVERY_KSTEP, prev[0])
+            ck.set_option(ck.OPT_STRAIGHT_LINE, prev[1])
+        assert ck.device_status() == 0
+        return dd.float().cpu().numpy()
+
+    # exact: small integers, every value representable in 16 bits (|sum| <= 4 * 64 = 256)
+    M, K = 520, 64
+    a = ck.fill_int(dt, (M, K), 171, 0, -2, 2)
+    bt = ck.fill_int(dt, (N, K), 171, 1, -2, 2)
+    want = (G.as_f64(is_bf, a) @ G.as_f64(is_bf, bt).T).astype(np.float32)
+    for cus in (256, 2):          # one tile per workgroup, and several (the next tile's waits count the stores)
+        for schedule in (1, 0):
+            assert np.array_equal(run(a, bt, None, 1.0, 0.0, M, K, cus, schedule), want), (cus, schedule)
+    assert np.array_equal(run(a, bt, None, -0.5, 0.0, M, K, 3), -0.5 * want)
+    # a one-hot Bt copies columns of A: position errors cannot cancel
+    K = 1024
+    a = ck.fill_uniform(dt, (M, K), 172, 0)
+    eye = np.zeros((N, K), dtype=np.float32)
+    eye[np.arange(N), (np.arange(N) * 7 + 5) % K] = 1.0
+    eye = G.f32_to_bf16_bits(eye) if is_bf else eye.astype(np.float16)
+    af = G.bf16_bits_to_f32(a) if is_bf else a.astype(np.float32)
+    assert np.array_equal(run(a, eye, None, 1.0, 0.0, M, K, 4), af[:, (np.arange(N) * 7 + 5) % K])
+    # random operands, long K, several tiles per workgroup: the same bits as the general fused kernel, with
+    # and without a C operand, and the oracle's fp32 result rounded once (at most 1 ulp apart)
+    bt = ck.fill_uniform(dt, (N, K), 172, 1)
+    c16 = ck.fill_uniform(dt, (M, N), 172, 2)
+    cf = G.bf16_bits_to_f32(c16) if is_bf else c16.astype(np.float32)
+    for c, alpha, beta in ((None, 1.0, 0.0), (c16, 0.75, -1.25)):
+        got = run(a, bt, c, alpha, beta, M, K, 3)
+        assert np.array_equal(got, run(a, bt, c, alpha, beta, M, K, 3, straight_line=0))
+        ref = oracle.gemm(odt, a, bt, None if c is None else cf, alpha, beta)
+        assert_close(oracle, ref, got)
+        ref16 = torch.from_numpy(ref).to(tdt).float().numpy()
+        assert np.all(np.abs(got - ref16) <= np.abs(ref16) * (2.0 ** -7 if is_bf else 2.0 ** -10) + 1e-3)
+
+
 def test_straight_line_kernel_headline_size_properties(ck):
     # 8192^3 in the headline configuration: constant operands have a closed form (every output
     # alpha * 10 * K), and a one-hot Bt picks columns of A exactly
