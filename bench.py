@@ -86,7 +86,8 @@ def sweep(ck, torch, args, ckdt, da, db, dd, M, N, K, cus, stream):
     for tile, c in ((256, 8), (128, 8), (128, 4), (64, 8), (64, 4)):
         wtr = ck.get_warp_tile_rows(tile, c)
         wave_rows = (wtr * 16, ck.get_num_acc(tile, c) // wtr * 16)
-        for segk, stages, p in ((32, 5, 0), (32, 4, 0), (64, 2, 0), (128, 2, 0), (64, 2, 2), (64, 2, 4), (32, 4, 4), (64, 4, 2), (64, 4, 4), (128, 2, 2)):
+        for segk, stages, p in ((32, 5, 0), (32, 4, 0), (64, 2, 0), (128, 2, 0), (64, 2, 2), (64, 2, 4), (32, 4, 4), (64, 4, 2), (64, 4, 4), (128, 2, 2),
+                                 (64, 1, 2)):   # one stage: loads and MFMAs alternate, the no-pipeline partner
             tuples.append((tile, segk, 0, 0, tile, tile, args.group, stages, p, c))
         if tile >= 128:   # the finer synchronisation granularities of port_1 / port_2 (producer/consumer kernels only)
             tuples.append((tile, 64, 2, 1, wave_rows[0], wave_rows[1], args.group, 2 if tile == 256 else 4, 2, c))
