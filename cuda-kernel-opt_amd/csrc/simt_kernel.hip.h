@@ -80,7 +80,7 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
     // slice: 240-256 registers for the 32- and 64-accumulator micro-tiles (1-2 waves per SIMD), spills with
     // 1024 threads (128 registers each). 8 steps keep those at 64-120 registers, 4 and more waves per SIMD
     // (fp32 4096^3, 128 tile, 32 accumulators: 90 TFLOP/s against 70); the small tile is better unrolled whole.
-    constexpr int K_UNROLL = NT >= 1024 ? 4 : (TILE == 32 ? KT : 8);
+        constexpr int K_UNROLL = NT >= 1024 ? 4 : (TILE == 32 ? KT : 8);
 
     extern __shared__ __attribute__((aligned(16))) char ck_simt_smem[];
     ACC* lds = reinterpret_cast<ACC*>(ck_simt_smem);
@@ -97,11 +97,31 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
     const int64_t m0 = (int64_t)blockIdx.x * TILE, n0 = (int64_t)blockIdx.y * TILE;
     const int K = g.K, N = g.N;
 
-    ACC acc[RM][RN];
+    // Register banks. A v_fmac_f32 whose three registers lie in the same bank (register number mod 4) issues
+    // at half rate (register-only loops on this chip: 71 TFLOP/s with all three in one bank, 137-147 with any
+    // other placement), and the allocator's natural layout puts a fifth of the multiply-adds there (the
+    // accumulators of a row and the B values are both runs of four, so column j of each lands in the same bank).
+    // A B value arrives in a 16-byte LDS read, an even-aligned run of four registers, so column j sits in bank
+    // base + j with an even base. Accumulator rows are therefore kept as even-aligned runs of four as well (the
+    // empty asm below pins them to such a run at the top of every slice), with column j stored in element j + 1:
+    // base_acc + j + 1 and base_b + j then always differ, whatever the A register is.
+    constexpr bool ROT = RN % 4 == 0;
+    constexpr int RG = ROT ? RN / 4 : 1;          // register quads per accumulator row
+    typedef ACC acc4_t __attribute__((ext_vector_type(4)));
+    acc4_t accq[RM][RG];
+    ACC accs[ROT ? 1 : RM][ROT ? 1 : RN];
+    auto acc_get = [&](int i, int j) -> ACC {
+        if constexpr (ROT) return accq[i][j / 4][(j + 1) & 3];
+        else return accs[i][j];
+    };
+    auto acc_set = [&](int i, int j, ACC v) {
+        if constexpr (ROT) accq[i][j / 4][(j + 1) & 3] = v;
+        else accs[i][j] = v;
+    };
 #pragma unroll
     for (int i = 0; i < RM; ++i)
 #pragma unroll
-        for (int j = 0; j < RN; ++j) acc[i][j] = (ACC)0;
+        for (int j = 0; j < RN; ++j) acc_set(i, j, (ACC)0);
 
     ACC ra[IT_RK][VEC], rb[IT_B][VEC];
 
@@ -161,28 +181,51 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
         }
     };
 
+    // CK_PROBE_SIMT_NOSTASH / CK_PROBE_SIMT_NOLDS: measurement builds only (wrong results): the loop without
+    // the global loads and LDS writes of the next slice / with one LDS read per slice instead of one per k.
     fetch(0);
     stash(0);
     __syncthreads();
     int buf = 0;
     for (int k0 = 0; k0 < K; k0 += KT) {
         const bool more = k0 + KT < K;
+#ifndef CK_PROBE_SIMT_NOSTASH
         if (more) fetch(k0 + KT);
+#endif
+        if (ROT) {
+#pragma unroll
+            for (int i = 0; i < RM; ++i)
+#pragma unroll
+                for (int q = 0; q < RG; ++q) asm volatile("" : "+v"(accq[i][q]));
+        }
         const ACC* as = a_s(buf) + ty * RM;
         const ACC* bs = b_s(buf) + tx * RN;
+#ifdef CK_PROBE_SIMT_NOLDS
+        ACC av[RM], bv[RN];
+#pragma unroll
+        for (int i = 0; i < RM; ++i) av[i] = as[i];
+#pragma unroll
+        for (int j = 0; j < RN; ++j) bv[j] = bs[j];
+#endif
 #pragma unroll(K_UNROLL)
         for (int k = 0; k < KT; ++k) {
+#ifndef CK_PROBE_SIMT_NOLDS
             ACC av[RM], bv[RN];
 #pragma unroll
             for (int i = 0; i < RM; ++i) av[i] = as[k * LD + i];
 #pragma unroll
             for (int j = 0; j < RN; ++j) bv[j] = bs[k * LD + j];
+#else
+            asm volatile("" ::: "memory");
+#endif
 #pragma unroll
             for (int i = 0; i < RM; ++i)
 #pragma unroll
-                for (int j = 0; j < RN; ++j) acc[i][j] = SimtIo<DT>::mad(av[i], bv[j], acc[i][j]);
+                for (int j = 0; j < RN; ++j) acc_set(i, j, SimtIo<DT>::mad(av[i], bv[j], acc_get(i, j)));
         }
+#ifndef CK_PROBE_SIMT_NOSTASH
         if (more) stash(buf ^ 1);
+#endif
         __syncthreads();
         buf ^= 1;
     }
@@ -191,7 +234,7 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
     for (int i = 0; i < RM; ++i) {
         DT* crow = C + (m0 + ty * RM + i) * N + n0 + tx * RN;
 #pragma unroll
-        for (int j = 0; j < RN; ++j) crow[j] = SimtIo<DT>::out(acc[i][j]);
+        for (int j = 0; j < RN; ++j) crow[j] = SimtIo<DT>::out(acc_get(i, j));
     }
 }
 
