@@ -228,3 +228,35 @@ def test_suggested_tunings_are_legal_and_follow_the_measured_rules(ck):
     assert picks(8192, 8192, 8200)["num_producer_warps"] == 2 and picks(8192, 8192, 8200)["tile_dim"] == 256  # K % 64 != 0
     with pytest.raises(ck.CkoptError):
         ck.suggest_gemm_tuning(0, 1, 1)
+
+
+def test_matmul_shmem_multiply_adds_avoid_one_bank_operands(tmp_path):
+    """A v_fmac_f32 whose three registers lie in one register bank (number mod 4) issues at half rate on
+    gfx950. The kernel keeps accumulator rows as aligned runs of four, rotated by one against the run of
+    four a 16-byte LDS read delivers, so no multiply-add of an instance with a four-wide row may have all
+    three in one bank. Checked on the compiled code of the kernel's own translation unit."""
+    import importlib.util
+    import subprocess
+    spec = importlib.util.spec_from_file_location("ckopt_build", os.path.join(ROOT, "cuda-kernel-opt_amd", "build.py"))
+    b = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(b)
+    src = os.path.join(ROOT, "cuda-kernel-opt_amd", "csrc", "simt_launch.hip")
+    out = str(tmp_path / "simt.s")
+    flags = [f for f in b.DEVICE_FLAGS if f != "-fPIC"]
+    r = subprocess.run([b.HIPCC] + flags + ["-S", "--cuda-device-only", src, "-o", out], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    text = open(out).read()
+    names = re.findall(r"^(_ZN2ck19matmul_shmem_kernelIfLi(\d+)ELi(\d+)ELi(\d+)ELb[01]EEEvNS_8SimtArgsE):", text, re.M)
+    assert len(names) >= 20
+    checked = 0
+    for name, tile, rm, rn in names:
+        if int(rn) % 4:
+            continue
+        body = text[text.index("\n" + name + ":"):]
+        body = body[:body.index("s_endpgm")]
+        ops = re.findall(r"v_fmac_f32_e32 v(\d+), v(\d+), v(\d+)", body)
+        assert len(ops) >= int(rm) * int(rn)
+        bad = [o for o in ops if int(o[0]) % 4 == int(o[1]) % 4 == int(o[2]) % 4]
+        assert not bad, "%s: %d of %d multiply-adds with all registers in one bank" % (name, len(bad), len(ops))
+        checked += 1
+    assert checked >= 10
