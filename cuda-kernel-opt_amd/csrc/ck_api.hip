@@ -117,6 +117,19 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ ws, int slices, l
     }
 }
 
+// The fp32 form of the same pass with four elements per thread (16-byte loads and stores): same additions in
+// the same order per element. For count % 4 == 0 and C, D on 16-byte boundaries.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__global__ void splitk_reduce4_kernel(const f32x4* __restrict__ ws, int slices, long long count4, const f32x4* C, f32x4* D, float alpha, float beta) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < count4; i += (long long)gridDim.x * blockDim.x) {
+        f32x4 sum = __builtin_nontemporal_load(ws + i);
+        for (int s = 1; s < slices; ++s) sum += __builtin_nontemporal_load(ws + (long long)s * count4 + i);
+        f32x4 v = alpha * sum;
+        if (beta != 0.f) v += C[i] * beta;
+        D[i] = v;
+    }
+}
+
 int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
                 int N, int K, const ck::GemmTuning& t, void* stream, int out16);
 
@@ -229,7 +242,13 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p, bek) : launch_gemm_stream_bf16(dim3(pgrid), s, p, bek);
             if (e == hipSuccess) {
                 const unsigned blocks = (unsigned)((count + 255) / 256 < 65535 * 8 ? (count + 255) / 256 : 65535 * 8);
-                if (!out16) hipLaunchKernelGGL((splitk_reduce_kernel<0, false>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
+                const bool vec4 = !out16 && count % 4 == 0 && ((uintptr_t)D | (uintptr_t)(beta != 0.f ? C : nullptr)) % 16 == 0;
+                if (vec4) {
+                    const long long count4 = count / 4;
+                    const unsigned b4 = (unsigned)((count4 + 255) / 256 < 65535 * 8 ? (count4 + 255) / 256 : 65535 * 8);
+                    hipLaunchKernelGGL(splitk_reduce4_kernel, dim3(b4), dim3(256), 0, s, reinterpret_cast<const f32x4*>(ws), slices, count4,
+                                       static_cast<const f32x4*>(C), static_cast<f32x4*>(D), alpha, beta);
+                } else if (!out16) hipLaunchKernelGGL((splitk_reduce_kernel<0, false>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
                 else if (dtype == CK_DT_F16) hipLaunchKernelGGL((splitk_reduce_kernel<1, false>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
                 else hipLaunchKernelGGL((splitk_reduce_kernel<1, true>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
                 e = hipGetLastError();
