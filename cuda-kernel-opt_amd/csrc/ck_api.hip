@@ -64,10 +64,17 @@ int status_ptr_for_current_device(unsigned int** out) {
 // Copies `rows` rows of K 2-byte elements into rows of Kp >= K elements (Kp % 8 == 0), zero filling
 // the tail: the form the direct-to-LDS loads need (every row starts on a 16-byte boundary). One
 // thread produces one 16-byte chunk of the destination from eight 2-byte reads.
-__global__ void pad_rows_kernel(const unsigned short* __restrict__ src, unsigned short* __restrict__ dst, int rows, int K, int Kp) {
+// Both operands go through one launch: chunks [0, rows_a * Kp / 8) belong to A, the rest to Bt.
+__global__ void pad_rows_kernel(const unsigned short* __restrict__ src_a, unsigned short* __restrict__ dst_a, int rows_a,
+                                const unsigned short* __restrict__ src_b, unsigned short* __restrict__ dst_b, int rows_b, int K, int Kp) {
     const int chunks_per_row = Kp / 8;
-    const long long total = (long long)rows * chunks_per_row;
-    for (long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x; c < total; c += (long long)gridDim.x * blockDim.x) {
+    const long long total_a = (long long)rows_a * chunks_per_row;
+    const long long total = total_a + (long long)rows_b * chunks_per_row;
+    for (long long cc = (long long)blockIdx.x * blockDim.x + threadIdx.x; cc < total; cc += (long long)gridDim.x * blockDim.x) {
+        const bool second = cc >= total_a;
+        const unsigned short* src = second ? src_b : src_a;
+        unsigned short* dst = second ? dst_b : dst_a;
+        const long long c = second ? cc - total_a : cc;
         const int r = (int)(c / chunks_per_row), k0 = (int)(c % chunks_per_row) * 8;
         // The chunk's 16 source bytes start on a 2-byte boundary: five aligned 4-byte words cover them,
         // shifted by two bytes where the start is odd. A word that lies only half inside
@@ -162,8 +169,8 @@ int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const void* C
     unsigned short* pb = pa + (size_t)M * Kp;
     const int threads = 256;
     auto blocks = [&](long long chunks) { long long b = (chunks + threads - 1) / threads; return (unsigned)(b < 65535 * 8 ? (b > 0 ? b : 1) : 65535 * 8); };
-    hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks((long long)M * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(A), pa, M, K, Kp);
-    hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks((long long)N * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(Bt), pb, N, K, Kp);
+    hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks(((long long)M + N) * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(A), pa, M,
+                       static_cast<const unsigned short*>(Bt), pb, N, K, Kp);
     int rc = hipGetLastError() == hipSuccess ? CK_OK : CK_ERR_HIP;
     if (rc == CK_OK) rc = gemm_launch(dtype, pa, pb, C, D, alpha, beta, M, N, Kp, t, stream, out16);
     if (hipFreeAsync(ws, s) != hipSuccess && rc == CK_OK) rc = CK_ERR_HIP;
