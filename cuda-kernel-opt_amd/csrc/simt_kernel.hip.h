@@ -105,17 +105,19 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
     // base + j with an even base. Accumulator rows are therefore kept as even-aligned runs of four as well (the
     // empty asm below pins them to such a run at the top of every slice), with column j stored in element j + 1:
     // base_acc + j + 1 and base_b + j then always differ, whatever the A register is.
-    constexpr bool ROT = RN % 4 == 0;
-    constexpr int RG = ROT ? RN / 4 : 1;          // register quads per accumulator row
-    typedef ACC acc4_t __attribute__((ext_vector_type(4)));
-    acc4_t accq[RM][RG];
+    // Rows of two columns: the same with pairs (an 8-byte LDS read delivers an even-aligned pair).
+    constexpr bool ROT = RN % 2 == 0;
+    constexpr int VW = RN % 4 == 0 ? 4 : 2;       // registers per aligned run
+    constexpr int RG = ROT ? RN / VW : 1;         // runs per accumulator row
+    typedef ACC accv_t __attribute__((ext_vector_type(VW)));
+    accv_t accq[RM][RG];
     ACC accs[ROT ? 1 : RM][ROT ? 1 : RN];
     auto acc_get = [&](int i, int j) -> ACC {
-        if constexpr (ROT) return accq[i][j / 4][(j + 1) & 3];
+        if constexpr (ROT) return accq[i][j / VW][(j + 1) % VW];
         else return accs[i][j];
     };
     auto acc_set = [&](int i, int j, ACC v) {
-        if constexpr (ROT) accq[i][j / 4][(j + 1) & 3] = v;
+        if constexpr (ROT) accq[i][j / VW][(j + 1) % VW] = v;
         else accs[i][j] = v;
     };
 #pragma unroll
