@@ -18,6 +18,7 @@ LIB_PATH = os.environ.get("CKOPT_LIB") or os.path.join(HERE, "lib", "libckopt.so
 DT_F16, DT_BF16, DT_F32, DT_I32 = 0, 1, 2, 3
 OK, ERR_BAD_PARAM, ERR_LDS_BUDGET, ERR_NO_INSTANCE, ERR_HIP, ERR_ALIGNMENT, ERR_NULL, ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6, -7
 OPT_SWIZZLE, OPT_SPIN_LIMIT, OPT_NUM_XCD, OPT_PRIO_MODE, OPT_PRODUCER_NAP, OPT_TILE_SYNC_BARRIER, OPT_STRAIGHT_LINE, OPT_SPLIT_K, OPT_BARRIER_EVERY_KSTEP = 0, 1, 2, 3, 4, 5, 6, 7, 8
+OPT_EVEN_ROUNDS = 9
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(

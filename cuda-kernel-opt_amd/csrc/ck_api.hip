@@ -39,6 +39,7 @@ std::atomic<int> g_prio_mode{0};
 std::atomic<int> g_producer_nap{0};
 std::atomic<int> g_tile_sync_barrier{0};
 std::atomic<int> g_straight_line{1};
+std::atomic<int> g_even_rounds{1};
 std::atomic<int> g_split_k{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
 std::atomic<int> g_barrier_every_kstep{1};
 constexpr int SPLIT_K_MIN_SLICE = 1024;  // shortest K slice split-K will make (shorter ones lose more in the reduction pass than they gain)
@@ -140,6 +141,20 @@ __global__ void splitk_reduce4_kernel(const f32x4* __restrict__ ws, int slices, 
 int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
                 int N, int K, const ck::GemmTuning& t, void* stream, int out16);
 
+// Workgroups of the persistent grid. With more tiles than CUs, num_cus workgroups run ceil(tiles / num_cus)
+// rounds and the last one is partly empty: CUs idle at the end while the full rounds before it ran at the
+// power-limited clock. The same number of rounds over fewer workgroups (whole XCDs' worth) keeps every round
+// full and spreads the power budget over fewer CUs (bf16 6143 x 4097 x 3071, 408 tiles: 208 workgroups x 2
+// rounds are 5.7 % faster than 256 + 152). Never more rounds than num_cus workgroups would take.
+int persistent_grid(int64_t tiles, int num_cus, int num_xcd, bool even_rounds) {
+    if (tiles <= num_cus) return (int)tiles;
+    if (!even_rounds) return num_cus;
+    const int64_t rounds = (tiles + num_cus - 1) / num_cus;
+    int64_t g = (tiles + rounds - 1) / rounds;
+    if (num_xcd > 1) g = (g + num_xcd - 1) / num_xcd * num_xcd;
+    return (int)(g < num_cus ? g : num_cus);
+}
+
 // Number of K slices the straight-line kernel uses for `tiles` 256 x 256 tiles (1: no split). policy 0: never;
 // 1: automatic - fewer tiles than half the CUs and at least four legal slices (two gain less than the
 // reduction pass costs); >= 2: that many slices if legal, else the next smaller legal count. Legal: whole XCD
@@ -221,7 +236,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     if (src != CK_OK) return src;
 
     const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
-    const int grid = (int)(tiles < t.num_cus ? tiles : t.num_cus);
+    const int grid = persistent_grid(tiles, t.num_cus, a.num_xcd, g_even_rounds.load() != 0);
     const dim3 block((t.num_producer_waves + t.num_consumer_waves) * WAVE);
     const size_t lds = (size_t)gemm_lds_bytes(t);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -473,6 +488,7 @@ int ckopt_set_option(int key, int value) {
         case 6: return g_straight_line.exchange(value != 0);
         case 7: if (value < 0 || value > 16) return ck::CK_ERR_BAD_PARAM; return g_split_k.exchange(value);
         case 8: return g_barrier_every_kstep.exchange(value != 0);
+        case 9: return g_even_rounds.exchange(value != 0);
         default: return ck::CK_ERR_BAD_PARAM;
     }
 }

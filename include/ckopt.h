@@ -169,6 +169,10 @@ int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, do
  *        body spread over both (three k-steps to land); 0: one barrier per two k-steps, all loads behind it (two
  *        k-steps to land) - 1.5 % faster at 8192^3 on random operand values (power-limited clock), slower wherever
  *        memory latency is higher (16384^3: 7 %, split-K: 12 %) or the clock is not power-limited (3 %).
+ * key 9: even rounds (default 1). A launch with more tiles than num_sms runs ceil(tiles / num_sms) rounds; with 1 the
+ *        persistent grid is the smallest number of workgroups (a multiple of the XCD count, at most num_sms) that
+ *        needs no more rounds, so that no round is partly empty (408 tiles on 256 CUs: 208 workgroups x 2 rounds
+ *        instead of 256 + 152; 5.7 % faster where the clock is power-limited); 0: always min(tiles, num_sms).
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

@@ -517,6 +517,34 @@ def test_straight_line_kernel_bit_exact(ck, M, N, K, cus, group):
             assert np.array_equal(got, want), every_kstep
 
 
+@pytest.mark.parametrize("M,N,K,cus", [
+    (1280, 1280, 192, 24),   # 25 tiles on 24 workgroups: 2 rounds, even rounds take 16 workgroups
+    (1279, 1025, 320, 12),   # ragged, 25 tiles on 12: 3 rounds, 9 -> 12 workgroups (rounded up to whole XCDs, capped)
+    (2304, 2048, 128, 40),   # 72 tiles on 40: 2 rounds of 36 -> 40
+])
+def test_even_rounds_grid_gives_the_same_result(ck, M, N, K, cus):
+    """The persistent grid with even rounds (fewer workgroups, same number of rounds) against min(tiles, num_sms):
+    exact small-integer products, both kernels' tile loops."""
+    a = ck.fill_int(ck.DT_F16, (M, K), 17, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 17, 1, -2, 2)
+    want = (G.as_f64(False, a) @ G.as_f64(False, bt).T).astype(np.float32)
+    tunings = [_straight_line_tuning(ck, cus, 4)]
+    if K % 64 == 0:
+        general = make_tuning(ck, 128, 64, 2, 2, 8)   # producer/consumer kernel, 128 x 128 tiles
+        general["num_sms"] = cus
+        general["tile_group_m"] = 3
+        tunings.append(general)
+    for t in tunings:
+        assert legal(ck, t)
+        for even in (0, 1):
+            prev = ck.set_option(ck.OPT_EVEN_ROUNDS, even)
+            try:
+                got = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+            finally:
+                ck.set_option(ck.OPT_EVEN_ROUNDS, prev)
+            assert np.array_equal(got, want), (even, t)
+
+
 def test_straight_line_kernel_epilogue_and_general_kernel_agree(ck, oracle):
     # beta != 0 (the epilogue reads C: the store accounting of the waits is off), 16-bit C/D, and the
     # same launches through the general fused kernel (option 6 off) give the same bits

@@ -204,6 +204,8 @@ def test_option_keys_reject_values_outside_their_range(ck):
     assert ck.set_option(ck.OPT_SPLIT_K, prev) == 0
     prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
     assert ck.set_option(ck.OPT_STRAIGHT_LINE, prev) == 0
+    prev = ck.set_option(ck.OPT_EVEN_ROUNDS, 0)
+    assert prev == 1 and ck.set_option(ck.OPT_EVEN_ROUNDS, prev) == 0
 
 
 def test_suggested_tunings_are_legal_and_follow_the_measured_rules(ck):
