@@ -80,7 +80,7 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
     // slice: 240-256 registers for the 32- and 64-accumulator micro-tiles (1-2 waves per SIMD), spills with
     // 1024 threads (128 registers each). 8 steps keep those at 64-120 registers, 4 and more waves per SIMD
     // (fp32 4096^3, 128 tile, 32 accumulators: 90 TFLOP/s against 70); the small tile is better unrolled whole.
-        constexpr int K_UNROLL = NT >= 1024 ? 4 : (TILE == 32 ? KT : 8);
+    constexpr int K_UNROLL = NT >= 1024 ? 4 : (TILE == 32 ? KT : 8);
 
     extern __shared__ __attribute__((aligned(16))) char ck_simt_smem[];
     ACC* lds = reinterpret_cast<ACC*>(ck_simt_smem);
