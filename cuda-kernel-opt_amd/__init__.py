@@ -31,6 +31,8 @@ _lib.ckopt_gemm_shmem_tc_async_opt_port_2.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_lp.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_lp.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2_noalloc.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2_noalloc.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_1.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_1.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 12 + [_p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_0.restype = _i
@@ -75,7 +77,8 @@ _lib.ckopt_error_string.restype = ctypes.c_char_p
 _lib.ckopt_error_string.argtypes = [_i]
 
 EXPORTED_SYMBOLS = [
-    "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_2_lp", "ckopt_gemm_shmem_tc_async_opt_port_1",
+    "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_2_lp", "ckopt_gemm_shmem_tc_async_opt_port_2_noalloc",
+    "ckopt_gemm_shmem_tc_async_opt_port_1",
     "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
     "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks", "ckopt_probe_counters",
@@ -173,6 +176,20 @@ def gemm_shmem_tc_async_opt_port_lp(dtype, A, B, C, D, alpha, beta, M, N, K, til
         dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
         bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
         num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port <DT, DT>")
+
+
+NOALLOC_SCRATCH_BYTES = 64 << 20
+
+
+def gemm_shmem_tc_async_opt_port_noalloc(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+                                         bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages,
+                                         num_producer_warps, num_consumer_warps, num_sms, stream=None):
+    """The port_2 launcher for callers that cannot allocate: operand copies and split-K planes in the library's
+    static device array of NOALLOC_SCRATCH_BYTES; raises CkoptError(ERR_TOO_LARGE) beyond it."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_2_noalloc(
+        dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+        bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+        num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port (no allocation)")
 
 
 def gemm_shmem_tc_async_opt_port_1(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_step_rows_a,

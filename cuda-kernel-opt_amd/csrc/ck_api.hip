@@ -30,6 +30,14 @@ hipError_t launch_matmul_shmem(int dtype, int tile, int accs, bool bt, dim3 grid
 // One status word per device; the kernels OR a bit into it when a bounded flag wait gives up.
 __device__ unsigned int ck_status_word[8 + 16 * 8] = {};  // [8..]: per-wave cycle counters of measurement builds
 
+// Scratch memory of the entry point that allocates nothing (ckopt_gemm_shmem_tc_async_opt_port_2_noalloc): the
+// zero-padded operand copies and the split-K planes of one launch. Every device the library runs on holds its own
+// copy of the array, at its own address, until the process ends. Host code never uses the array's name as an
+// address: the per-device address comes from hipGetSymbolAddress (static_scratch_for_current_device below). That
+// host-side use is what makes the compiler emit the array into the code object under a global symbol the runtime can
+// look up; marked __attribute__((used)) it would stay a local symbol and the lookup would abort the process.
+static __device__ __align__(256) unsigned char scratch[CKOPT_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 std::atomic<int> g_swizzle{1};
@@ -59,6 +67,23 @@ int status_ptr_for_current_device(unsigned int** out) {
         g_status_ptr[dev] = static_cast<unsigned int*>(p);
     }
     *out = g_status_ptr[dev];
+    return ck::CK_OK;
+}
+
+unsigned char* g_scratch_ptr[MAX_DEV] = {};
+
+// Device address of this device's copy of `scratch`, looked up once per device with that device current.
+int static_scratch_for_current_device(unsigned char** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return ck::CK_ERR_HIP;
+    if (dev < 0 || dev >= MAX_DEV) return ck::CK_ERR_HIP;
+    std::lock_guard<std::mutex> lock(g_status_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return ck::CK_ERR_HIP;
+        g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+    }
+    *out = g_scratch_ptr[dev];
     return ck::CK_OK;
 }
 
@@ -138,8 +163,44 @@ __global__ void splitk_reduce4_kernel(const f32x4* __restrict__ ws, int slices, 
     }
 }
 
+// Where a launch takes device memory beyond its operands from (the zero-padded operand copies, the split-K planes).
+// ALLOCATE: stream-ordered allocations inside the call. PROVIDED: the buffer [ptr, ptr + bytes) that the caller or the
+// library's static array supplies; pieces are carved off its front on 256-byte boundaries and nothing is allocated.
+struct Scratch {
+    enum Mode { ALLOCATE, PROVIDED } mode;
+    char* ptr;
+    size_t bytes;
+};
+constexpr size_t SCRATCH_ALIGN = 256;
+size_t scratch_round(size_t n) { return (n + SCRATCH_ALIGN - 1) / SCRATCH_ALIGN * SCRATCH_ALIGN; }
+
+// Takes `need` bytes: CK_OK with *out set, CK_ERR_HIP if the allocation failed, CK_ERR_TOO_LARGE if a provided buffer
+// is too small. A piece of an ALLOCATE scratch is handed back with scratch_release().
+int scratch_take(Scratch& sc, size_t need, hipStream_t s, void** out) {
+    if (sc.mode == Scratch::ALLOCATE) {
+        *out = nullptr;
+        if (hipMallocAsync(out, need, s) != hipSuccess || !*out) {
+            (void)hipGetLastError();  // the failure is reported through the return value, not left for the next HIP call
+            return ck::CK_ERR_HIP;
+        }
+        return ck::CK_OK;
+    }
+    const uintptr_t base = (uintptr_t)sc.ptr;
+    const uintptr_t aligned = (base + SCRATCH_ALIGN - 1) / SCRATCH_ALIGN * SCRATCH_ALIGN;
+    const size_t skip = (size_t)(aligned - base);
+    if (!sc.ptr || skip > sc.bytes || need > sc.bytes - skip) return ck::CK_ERR_TOO_LARGE;
+    *out = (void*)aligned;
+    const size_t used = skip + scratch_round(need);
+    sc.ptr += used < sc.bytes ? used : sc.bytes;
+    sc.bytes -= used < sc.bytes ? used : sc.bytes;
+    return ck::CK_OK;
+}
+bool scratch_release(const Scratch& sc, void* piece, hipStream_t s) {
+    return sc.mode != Scratch::ALLOCATE || hipFreeAsync(piece, s) == hipSuccess;
+}
+
 int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
-                int N, int K, const ck::GemmTuning& t, void* stream, int out16);
+                int N, int K, const ck::GemmTuning& t, void* stream, int out16, Scratch sc);
 
 // Workgroups of the persistent grid. With more tiles than CUs, num_cus workgroups run ceil(tiles / num_cus)
 // rounds and the last one is partly empty: CUs idle at the end while the full rounds before it ran at the
@@ -173,13 +234,14 @@ int split_k_slices(int64_t tiles, int N, int K, int num_cus, int policy) {
 // K % 8 != 0 or operands off a 16-byte boundary: the product is computed from zero-padded,
 // aligned copies of A and Bt in a stream-ordered temporary (zeros in the K tail add nothing).
 int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta,
-                         int M, int N, int K, const ck::GemmTuning& t, void* stream, int out16) {
+                         int M, int N, int K, const ck::GemmTuning& t, void* stream, int out16, Scratch sc) {
     using namespace ck;
     const int Kp = (K + CHUNK_ELEMS - 1) / CHUNK_ELEMS * CHUNK_ELEMS;
     const size_t bytes_a = (size_t)M * Kp * 2, bytes_b = (size_t)N * Kp * 2;
     hipStream_t s = static_cast<hipStream_t>(stream);
     void* ws = nullptr;
-    if (hipMallocAsync(&ws, bytes_a + bytes_b, s) != hipSuccess || !ws) return CK_ERR_HIP;
+    const int trc = scratch_take(sc, bytes_a + bytes_b, s, &ws);
+    if (trc != CK_OK) return trc;
     unsigned short* pa = static_cast<unsigned short*>(ws);
     unsigned short* pb = pa + (size_t)M * Kp;
     const int threads = 256;
@@ -187,13 +249,13 @@ int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const void* C
     hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks(((long long)M + N) * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(A), pa, M,
                        static_cast<const unsigned short*>(Bt), pb, N, K, Kp);
     int rc = hipGetLastError() == hipSuccess ? CK_OK : CK_ERR_HIP;
-    if (rc == CK_OK) rc = gemm_launch(dtype, pa, pb, C, D, alpha, beta, M, N, Kp, t, stream, out16);
-    if (hipFreeAsync(ws, s) != hipSuccess && rc == CK_OK) rc = CK_ERR_HIP;
+    if (rc == CK_OK) rc = gemm_launch(dtype, pa, pb, C, D, alpha, beta, M, N, Kp, t, stream, out16, sc);
+    if (!scratch_release(sc, ws, s) && rc == CK_OK) rc = CK_ERR_HIP;
     return rc;
 }
 
 int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
-                int N, int K, const ck::GemmTuning& t, void* stream, int out16) {
+                int N, int K, const ck::GemmTuning& t, void* stream, int out16, Scratch sc) {
     using namespace ck;
     if (!(dtype == CK_DT_F16 || dtype == CK_DT_BF16)) return CK_ERR_BAD_PARAM;
     if (M <= 0 || N <= 0 || K <= 0) return CK_ERR_BAD_PARAM;
@@ -206,7 +268,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     if (((uintptr_t)D & elem_mask) || ((uintptr_t)C & elem_mask)) return CK_ERR_ALIGNMENT;
     // the kernels want every operand row on a 16-byte boundary
     if (K % CHUNK_ELEMS != 0 || ((uintptr_t)A & 15) || ((uintptr_t)Bt & 15))
-        return gemm_launch_repacked(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, out16);
+        return gemm_launch_repacked(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, out16, sc);
     // one tile's rows are addressed through a 32-bit buffer offset
     if ((int64_t)t.tile_dim * K * 2 >= (int64_t)1 << 31) return CK_ERR_TOO_LARGE;
 
@@ -248,13 +310,19 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         // Few tiles and a deep K: cut K into slices so that every CU has an item, partial products into
         // a stream-ordered workspace, one reduction pass.
         const bool bek = g_barrier_every_kstep.load() != 0;
-        const int slices = split_k_slices(tiles, N, K, t.num_cus, g_split_k.load());
+        int slices = split_k_slices(tiles, N, K, t.num_cus, g_split_k.load());
+        const long long count = (long long)M * N;
+        float* ws = nullptr;
+        if (slices > 1) {
+            const int trc = scratch_take(sc, (size_t)slices * count * sizeof(float), s, (void**)&ws);
+            // a provided buffer that is too small is the caller's error; a failed allocation is not: the
+            // single-pass launch computes the same product without any
+            if (trc == CK_ERR_TOO_LARGE) return trc;
+            if (trc != CK_OK) slices = 1;
+        }
         if (slices == 1) {
             e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a, bek) : launch_gemm_stream_bf16(dim3(grid), s, a, bek);
         } else {
-            const long long count = (long long)M * N;
-            float* ws = nullptr;
-            if (hipMallocAsync((void**)&ws, (size_t)slices * count * sizeof(float), s) != hipSuccess || !ws) return CK_ERR_HIP;
             GemmArgs p = a;
             p.split_k = slices;
             p.split_chunk = tiles < 32 ? (int)tiles : 32;
@@ -275,7 +343,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
                 else hipLaunchKernelGGL((splitk_reduce_kernel<1, true>), dim3(blocks), dim3(256), 0, s, ws, slices, count, C, D, alpha, beta);
                 e = hipGetLastError();
             }
-            if (hipFreeAsync(ws, s) != hipSuccess && e == hipSuccess) e = hipErrorUnknown;
+            if (!scratch_release(sc, ws, s) && e == hipSuccess) e = hipErrorUnknown;
         }
     } else if (t.num_producer_waves == 0) {
         e = dtype == CK_DT_F16 ? launch_gemm_fused_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a)
@@ -309,7 +377,7 @@ int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* B
                                          int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
     const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
                            tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0);
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0, Scratch{Scratch::ALLOCATE, nullptr, 0});
 }
 
 int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void* Bt, const void* C, void* D,
@@ -319,7 +387,21 @@ int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void
                                             int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
     const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
                            tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 1);
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 1, Scratch{Scratch::ALLOCATE, nullptr, 0});
+}
+
+int ckopt_gemm_shmem_tc_async_opt_port_2_noalloc(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                                 float alpha, float beta, int M, int N, int K, int tile_dim,
+                                                 int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                                                 int bar_step_rows_b, int tile_group_m, int num_stages,
+                                                 int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    unsigned char* ptr = nullptr;
+    const int rc = static_scratch_for_current_device(&ptr);
+    if (rc != ck::CK_OK) return rc;
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0,
+                       Scratch{Scratch::PROVIDED, reinterpret_cast<char*>(ptr), (size_t)CKOPT_NOALLOC_SCRATCH_BYTES});
 }
 
 int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
@@ -338,7 +420,7 @@ int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* B
     }
     const ck::GemmTuning t{tile_dim, segment_dim_k, sa, sb, bar_step_rows_a, bar_step_rows_b,
                            tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0);
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0, Scratch{Scratch::ALLOCATE, nullptr, 0});
 }
 
 int ckopt_gemm_shmem_tc_async_opt_port_0(int dtype, const void* A, const void* Bt, const float* C, float* D,
@@ -347,7 +429,7 @@ int ckopt_gemm_shmem_tc_async_opt_port_0(int dtype, const void* A, const void* B
                                          int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
     const ck::GemmTuning t{tile_dim, segment_dim_k, 0, 0, tile_dim, tile_dim,
                            tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0);
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0, Scratch{Scratch::ALLOCATE, nullptr, 0});
 }
 
 int ckopt_get_lds_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,

@@ -65,6 +65,23 @@ int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void
                                             int bar_step_rows_b, int tile_group_m, int num_stages,
                                             int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
 
+/* The port_2 launcher above for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose launcher needs no
+ * memory beyond its operands. Same parameters and results as ckopt_gemm_shmem_tc_async_opt_port_2 (the same kernels
+ * in the same order), but the zero-padded operand copies (K % 8 != 0 or operands off a 16-byte boundary:
+ * (M + N) * round_up(K, 8) * 2 bytes) and the split-K planes (slices * M * N * 4 bytes) live in a static device array
+ * of CKOPT_NOALLOC_SCRATCH_BYTES inside the library instead of stream-ordered allocations: no hipMalloc, hipFree or
+ * allocating library routine is called. A launch that needs more than the array holds (both pieces, each rounded up
+ * to 256 bytes) returns CKOPT_ERR_TOO_LARGE and D is not written; ckopt_set_option(7, 0) makes such a launch
+ * fit by not cutting K. Every device holds one array and every call on a device uses it: calls that overlap on one
+ * device (different streams, different threads) race on it. Nothing in it needs to start at zero. */
+#define CKOPT_NOALLOC_SCRATCH_BYTES (64u << 20)
+int ckopt_gemm_shmem_tc_async_opt_port_2_noalloc(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                                 float alpha, float beta, int M, int N, int K, int tile_dim,
+                                                 int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                                                 int bar_step_rows_b, int tile_group_m, int num_stages,
+                                                 int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
+
 /* Replaces gemm_shmem_tc_async_opt_port<DT,DT_ACC>() of matmul_shmem_tc_async_opt_port_1.cu:889-965:
  * every wave tile (or every 16-row block) has its own signal, i.e. port_2 with maximal bar_steps. */
 int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
