@@ -33,6 +33,10 @@ _lib.ckopt_gemm_shmem_tc_async_opt_port_2_lp.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_lp.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_noalloc.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_noalloc.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
+_lib.ckopt_gemm_workspace_bytes.restype = _i64
+_lib.ckopt_gemm_workspace_bytes.argtypes = [_i] * 15
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2_ws.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2_ws.argtypes = [_i, _i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p, ctypes.c_size_t, _p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_1.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_1.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 12 + [_p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_0.restype = _i
@@ -78,6 +82,7 @@ _lib.ckopt_error_string.argtypes = [_i]
 
 EXPORTED_SYMBOLS = [
     "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_2_lp", "ckopt_gemm_shmem_tc_async_opt_port_2_noalloc",
+    "ckopt_gemm_workspace_bytes", "ckopt_gemm_shmem_tc_async_opt_port_2_ws",
     "ckopt_gemm_shmem_tc_async_opt_port_1",
     "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
@@ -176,6 +181,27 @@ def gemm_shmem_tc_async_opt_port_lp(dtype, A, B, C, D, alpha, beta, M, N, K, til
         dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
         bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
         num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port <DT, DT>")
+
+
+def gemm_workspace_bytes(M, N, K, operands_aligned, tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
+                         bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms):
+    """Bytes of caller-owned workspace gemm_shmem_tc_async_opt_port_ws needs for this launch (0: none)."""
+    r = _lib.ckopt_gemm_workspace_bytes(M, N, K, int(bool(operands_aligned)), tile_dim, segment_dim_k, bar_steps_a, bar_steps_b,
+                                        bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+                                        num_consumer_warps, num_sms)
+    if r < 0:
+        raise CkoptError(int(r), "gemm_workspace_bytes")
+    return int(r)
+
+
+def gemm_shmem_tc_async_opt_port_ws(dtype, cd_dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+                                    bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages,
+                                    num_producer_warps, num_consumer_warps, num_sms, workspace, workspace_bytes, stream=None):
+    """The port_2 launcher on a caller-owned workspace (nothing is allocated); cd_dtype DT_F32 or the operands' type."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_2_ws(
+        dtype, cd_dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+        bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps,
+        num_sms, _dptr(workspace), int(workspace_bytes), _stream(stream)), "gemm_shmem_tc_async_opt_port (workspace)")
 
 
 NOALLOC_SCRATCH_BYTES = 64 << 20

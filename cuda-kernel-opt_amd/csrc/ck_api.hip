@@ -231,6 +231,27 @@ int split_k_slices(int64_t tiles, int N, int K, int num_cus, int policy) {
     return tiles * 2 <= num_cus && cand >= 4 ? cand : 1;
 }
 
+// Scratch bytes a launch takes from a provided buffer whose start is on a 256-byte boundary (the launcher's own
+// rules, evaluated without launching): the zero-padded operand copies when K % 8 != 0 or the operands are not on
+// 16-byte boundaries, then the split-K planes when the straight-line kernel cuts K.
+size_t scratch_need(int M, int N, int K, bool operands_aligned, const ck::GemmTuning& t) {
+    using namespace ck;
+    size_t need = 0;
+    int k = K;
+    if (K % CHUNK_ELEMS != 0 || !operands_aligned) {
+        k = (K + CHUNK_ELEMS - 1) / CHUNK_ELEMS * CHUNK_ELEMS;
+        need += scratch_round(((size_t)M + (size_t)N) * k * 2);
+    }
+    const bool straight_line = g_straight_line.load() && g_swizzle.load() && t.num_producer_waves == 0 && t.num_consumer_waves == 8 &&
+                               t.tile_dim == 256 && t.segment_dim_k == 32 && t.num_stages == 5 && k % STREAM_K_MULTIPLE_HOST == 0;
+    if (straight_line) {
+        const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+        const int slices = split_k_slices(tiles, N, k, t.num_cus, g_split_k.load());
+        if (slices > 1) need += scratch_round((size_t)slices * M * N * sizeof(float));
+    }
+    return need;
+}
+
 // K % 8 != 0 or operands off a 16-byte boundary: the product is computed from zero-padded,
 // aligned copies of A and Bt in a stream-ordered temporary (zeros in the K tail add nothing).
 int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta,
@@ -404,6 +425,30 @@ int ckopt_gemm_shmem_tc_async_opt_port_2_noalloc(int dtype, const void* A, const
                        Scratch{Scratch::PROVIDED, reinterpret_cast<char*>(ptr), (size_t)CKOPT_NOALLOC_SCRATCH_BYTES});
 }
 
+int64_t ckopt_gemm_workspace_bytes(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a,
+                                   int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
+                                   int num_producer_waves, int num_consumer_waves, int num_cus) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    if (M <= 0 || N <= 0 || K <= 0) return ck::CK_ERR_BAD_PARAM;
+    const int rc = ck::check_gemm_tuning(t);
+    if (rc != ck::CK_OK) return rc;
+    const size_t need = scratch_need(M, N, K, operands_aligned != 0, t);
+    return need ? (int64_t)(need + SCRATCH_ALIGN) : 0;  // room to start on a 256-byte boundary inside any buffer
+}
+
+int ckopt_gemm_shmem_tc_async_opt_port_2_ws(int dtype, int cd_dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim, int segment_dim_k,
+                                            int bar_steps_a, int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b,
+                                            int tile_group_m, int num_stages, int num_producer_waves, int num_consumer_waves,
+                                            int num_cus, void* workspace, size_t workspace_bytes, void* stream) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    if (!(cd_dtype == ck::CK_DT_F32 || cd_dtype == dtype)) return ck::CK_ERR_BAD_PARAM;
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, cd_dtype == ck::CK_DT_F32 ? 0 : 1,
+                       Scratch{Scratch::PROVIDED, static_cast<char*>(workspace), workspace ? workspace_bytes : 0});
+}
+
 int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
                                          float alpha, float beta, int M, int N, int K, int tile_dim,
                                          int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
@@ -480,7 +525,7 @@ int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out)
     static const int pc_256[10] = {256, 64, 0, 0, 256, 256, 4, 2, 2, 8};
     const int* pick = fused_64;
     const int64_t t256 = tiles(256);
-    const bool split_ok = kp % STREAM_K_MULTIPLE_HOST == 0 && split_k_slices(t256, N, kp, num_cus, 1) > 1;
+    const bool split_ok = kp % STREAM_K_MULTIPLE_HOST == 0 && split_k_slices(t256, N, kp, num_cus, g_split_k.load()) > 1;
     if (t256 * 2 >= num_cus) pick = kp % STREAM_K_MULTIPLE_HOST == 0 ? straight_line : pc_256;
     else if (split_ok) pick = straight_line;
     else if (tiles(128) * 2 >= num_cus) pick = fused_128;

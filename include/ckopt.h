@@ -8,12 +8,18 @@
  *     the error (matmul_shmem_tc_async_opt_port_2.cu:76-85, :1112-1123);
  *   - a trailing `stream` (a hipStream_t passed as void*, NULL = default stream) is added;
  *   - "warps" are 64-lane wavefronts and "SMs" are compute units.
- * All pointers are device memory owned by the caller. Nothing is allocated, freed or
- * synchronised; launches are asynchronous on `stream`.
+ * All pointers are device memory owned by the caller. Nothing is synchronised; launches are asynchronous on `stream`.
+ * Device memory beyond the operands is needed in two cases only (zero-padded operand copies when K % 8 != 0 or an
+ * operand is off a 16-byte boundary; partial planes when the straight-line kernel cuts K into slices). The reference's
+ * launcher needs none and allocates nothing (port_2.cu:1088-1168; its drivers own all memory, :1200-1203). Here the
+ * plain entry points take it from stream-ordered allocations on `stream` (hipMallocAsync / hipFreeAsync);
+ * ckopt_gemm_shmem_tc_async_opt_port_2_ws takes it from a workspace the caller owns and allocates nothing;
+ * ckopt_gemm_shmem_tc_async_opt_port_2_noalloc takes it from a static array inside the library.
  */
 #ifndef CKOPT_H
 #define CKOPT_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -64,6 +70,23 @@ int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void
                                             int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
                                             int bar_step_rows_b, int tile_group_m, int num_stages,
                                             int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
+
+/* The port_2 launcher (both C / D forms) on caller-owned scratch memory: the reference's ownership rule (the launcher
+ * works on the caller's device memory only, port_2.cu:1088-1168, :1200-1203) for the launches that need memory beyond
+ * the operands. cd_dtype is CKOPT_DT_F32 (the port_2 entry) or equal to dtype (the _lp entry). `workspace` is device
+ * memory of `workspace_bytes` bytes, any alignment, used only during the call's work on `stream`; it may be NULL when
+ * the launch needs none. ckopt_gemm_workspace_bytes returns how much the launch with these sizes and this tuning
+ * needs under the process's current options (0: none; negative: the error the launch would give);
+ * operands_aligned != 0 promises A and Bt on 16-byte boundaries. A workspace that is too small gives
+ * CKOPT_ERR_TOO_LARGE and D is not written; nothing is allocated in any case. */
+int64_t ckopt_gemm_workspace_bytes(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a,
+                                   int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
+                                   int num_producer_waves, int num_consumer_waves, int num_cus);
+int ckopt_gemm_shmem_tc_async_opt_port_2_ws(int dtype, int cd_dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim, int segment_dim_k,
+                                            int bar_steps_a, int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b,
+                                            int tile_group_m, int num_stages, int num_producer_waves, int num_consumer_waves,
+                                            int num_cus, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The port_2 launcher above for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose launcher needs no

@@ -287,45 +287,54 @@ def test_launch_is_deterministic_and_swizzle_is_transparent(ck):
     assert np.array_equal(d1.view(np.uint32), d3.view(np.uint32))
 
 
-# ---- full-size configurations: sampled rows against the oracle + exact integer identities ----------------
-def full_size_check(ck, oracle, dtype, odt, M, N, K, t, fill, rows):
+# ---- full-size configurations: the whole matrix against the oracle + exact integer identities --------------
+def full_size_check(ck, oracle, dtype, odt, M, N, K, tunings, fill):
+    """Every tuning's result against the blocked oracle over ALL rows (one oracle pass per configuration)."""
     a, bt = fill(0, (M, K)), fill(1, (N, K))
-    d = G.run_gemm(ck, dtype, a, bt, t=t)
-    for r0 in rows:
-        ref = oracle.gemm(odt, a, bt, rows=(r0, r0 + 8))
-        assert_close(oracle, ref, d[r0:r0 + 8])
-    assert np.isfinite(d).all()
-    # linearity checksum in float64: D @ 1 == A @ (Bt^T @ 1)
+    ref = oracle.gemm(odt, a, bt)
     bis16 = dtype == ck.DT_BF16
-    lhs = d.astype(np.float64).sum(axis=1)
     rhs = G.as_f64(bis16, a) @ G.as_f64(bis16, bt).sum(axis=0)
     scale = (np.abs(G.as_f64(bis16, a)) @ np.abs(G.as_f64(bis16, bt)).sum(axis=0)) + 1.0
-    assert np.max(np.abs(lhs - rhs) / scale) < 1e-4
+    for t in tunings:
+        d = G.run_gemm(ck, dtype, a, bt, t=t)
+        n, worst = oracle.count_outside_rel(ref, d, RTOL)
+        assert n == 0, "%d elements outside tolerance, worst ratio %g, tuning %s" % (n, worst, t)
+        # linearity checksum in float64: D @ 1 == A @ (Bt^T @ 1)
+        assert np.max(np.abs(d.astype(np.float64).sum(axis=1) - rhs) / scale) < 1e-4, t
+
+
+def suggested_tuning(ck, M, N, K, cus=256):
+    """The tuple bench.py times for this size (ckopt_suggest_gemm_tuning)."""
+    return dict(ck.suggest_gemm_tuning(M, N, K, cus))
 
 
 def test_config3_fp16_8192_headline(ck, oracle):
     M = N = K = 8192
-    t = make_tuning(ck, 256, 64, 2, 2, 8)
-    full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t,
-                    lambda s, shape: ck.fill_uniform(ck.DT_F16, shape, 0xC0FFEE03, s), rows=(0, 4000, 8184))
+    headline = suggested_tuning(ck, M, N, K)
+    assert (headline["tile_dim"], headline["segment_dim_k"], headline["num_stages"], headline["num_producer_warps"],
+            headline["num_consumer_warps"]) == (256, 32, 5, 0, 8)
+    pc = make_tuning(ck, 256, 64, 2, 2, 8)   # the reference's design: dedicated producer waves
+    full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, (headline, pc),
+                    lambda s, shape: ck.fill_uniform(ck.DT_F16, shape, 0xC0FFEE03, s))
     # exact: small integers at full size
     a = ck.fill_int(ck.DT_F16, (M, K), 0xC0FFEE03, 2, -1, 1)
     bt = ck.fill_int(ck.DT_F16, (N, K), 0xC0FFEE03, 3, -1, 1)
-    d = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
     ai, bi = a.astype(np.int64), bt.astype(np.int64)
-    assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
-    assert np.array_equal(d.astype(np.int64).sum(axis=0), bi @ ai.sum(axis=0))
-    assert np.array_equal(d[4095], (ai[4095] @ bi.T).astype(np.float32))
+    for t in (headline, pc):
+        d = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+        assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
+        assert np.array_equal(d.astype(np.int64).sum(axis=0), bi @ ai.sum(axis=0))
+        assert np.array_equal(d[4095], (ai[4095] @ bi.T).astype(np.float32))
 
 
 def test_config4_long_k_shift_sync_regime(ck, oracle):
     M = N = 2048
     K = 32768
     fill = lambda s, shape: ck.fill_normal(ck.DT_F16, shape, 0xC0FFEE04, s, 0.0, 0.1)
-    # the last tuple is the straight-line kernel: 64 tiles of 256 x 256, K cut into 4 slices + reduction pass
-    for t in (make_tuning(ck, 128, 64, 4, 4, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 4, 2),
-              make_tuning(ck, 128, 64, 4, 4, 8, "acc", 1, 3), make_tuning(ck, 256, 32, 5, 0, 8)):
-        full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t, fill, rows=(0, 1024))
+    # the first tuple is what bench.py times: the straight-line kernel, 64 tiles of 256 x 256, K cut into 4 slices
+    full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K,
+                    (suggested_tuning(ck, M, N, K), make_tuning(ck, 128, 64, 4, 4, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 4, 2),
+                     make_tuning(ck, 128, 64, 4, 4, 8, "acc", 1, 3)), fill)
 
 
 # ---- K not a multiple of 8 / operands off a 16-byte boundary: zero-padded repack in front of the kernel ----
@@ -360,13 +369,13 @@ def test_operands_off_16_byte_boundary(ck):
 
 
 def test_config5_bf16_6143x4097x3071(ck, oracle):
-    # every dimension ragged, rows of 3071 bf16 values (6142 bytes): sampled rows against the CPU
+    # every dimension ragged, rows of 3071 bf16 values (6142 bytes): the whole matrix against the CPU
     # oracle within the stated tolerance, and the row-sum identity over the whole result
     M, N, K = 6143, 4097, 3071
     fill = lambda s, shape: ck.fill_uniform(ck.DT_BF16, shape, 0xC0FFEE05, s)
-    for t in (make_tuning(ck, 256, 64, 2, 2, 8), make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 128, 64, 4, 4, 8, "wave", 2, 1),
-              make_tuning(ck, 256, 32, 5, 0, 8)):
-        full_size_check(ck, oracle, ck.DT_BF16, oracle.DT_BF16, M, N, K, t, fill, rows=(0, 3000, M - 8))
+    full_size_check(ck, oracle, ck.DT_BF16, oracle.DT_BF16, M, N, K,
+                    (suggested_tuning(ck, M, N, K), make_tuning(ck, 256, 64, 2, 2, 8), make_tuning(ck, 256, 64, 2, 0, 8),
+                     make_tuning(ck, 128, 64, 4, 4, 8, "wave", 2, 1)), fill)
     # exact at full size on small integers
     a = ck.fill_int(ck.DT_BF16, (M, K), 0xC0FFEE05, 2, -1, 1)
     bt = ck.fill_int(ck.DT_BF16, (N, K), 0xC0FFEE05, 3, -1, 1)
@@ -379,9 +388,8 @@ def test_config5_bf16_6143x4097x3071(ck, oracle):
 
 def test_fused_variant_full_size(ck, oracle):
     M = N = K = 8192
-    for t in (make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 256, 32, 5, 0, 8)):
-        full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, t,
-                        lambda s, shape: ck.fill_uniform(ck.DT_F16, shape, 0xC0FFEE03, s), rows=(0, 4000, 8184))
+    full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, (make_tuning(ck, 256, 64, 2, 0, 8), make_tuning(ck, 256, 32, 5, 0, 8)),
+                    lambda s, shape: ck.fill_uniform(ck.DT_F16, shape, 0xC0FFEE03, s))
 
 
 def test_inner_loop_ceiling_probe_runs(ck):
@@ -714,3 +722,168 @@ def test_straight_line_kernel_random_shapes(ck):
             ck.set_option(ck.OPT_BARRIER_EVERY_KSTEP, prev[0])
             ck.set_option(ck.OPT_SPLIT_K, prev[1])
         assert np.array_equal(got, want.astype(np.float32)), (case, M, N, K, cus, group, dt, beta, every_kstep, slices)
+
+
+# ---- split-K through every form of the reduction pass -----------------------------------------------------
+@pytest.mark.parametrize("dt_name", ["f16", "bf16"])
+@pytest.mark.parametrize("policy", [1, 4])          # automatic (8 slices for this shape) and four slices asked for
+@pytest.mark.parametrize("with_c", [False, True])
+def test_split_k_16_bit_output(ck, oracle, dt_name, policy, with_c):
+    # the <half, half> role on a shape that the straight-line kernel cuts along K: 4 tiles, K = 8192
+    dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16
+    odt = oracle.DT_F16 if dt_name == "f16" else oracle.DT_BF16
+    is_bf = dt_name == "bf16"
+    tdt = torch.bfloat16 if is_bf else torch.float16
+    M, N, K = 512, 512, 8192
+    t = _straight_line_tuning(ck)
+    alpha, beta = (2.0, -1.0) if with_c else (1.0, 0.0)
+
+    def to16(x32):
+        return torch.from_numpy(np.ascontiguousarray(x32, dtype=np.float32)).to(tdt)
+
+    def run(a, bt, c16, split):
+        da, db = G.to_dev(a), G.to_dev(bt)
+        dc = None if c16 is None else c16.cuda()
+        dd = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+        prev = ck.set_option(ck.OPT_SPLIT_K, split)
+        try:
+            ck.gemm_shmem_tc_async_opt_port_lp(dt, da, db, dc, dd, alpha, beta, M, N, K, t["tile_dim"], t["segment_dim_k"],
+                                               t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                               t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                               t["num_consumer_warps"], t["num_sms"])
+        finally:
+            ck.set_option(ck.OPT_SPLIT_K, prev)
+        assert ck.device_status() == 0
+        return dd.cpu()
+
+    # small integers: every partial sum is exact in fp32, so slices and single pass round the same number once
+    a = ck.fill_int(dt, (M, K), 181, 0, -2, 2)
+    bt = ck.fill_int(dt, (N, K), 181, 1, -2, 2)
+    c16 = to16(ck.fill_int(ck.DT_F32, (M, N), 181, 2, -3, 3)) if with_c else None
+    exact = alpha * (G.as_f64(is_bf, a) @ G.as_f64(is_bf, bt).T)
+    if with_c:
+        exact = exact + beta * c16.double().numpy()
+    want = to16(exact)   # |exact| < 2^24: the float32 step is exact, one rounding to 16 bits
+    got = run(a, bt, c16, policy)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(got.view(torch.int16), run(a, bt, c16, 0).view(torch.int16))
+    # uniform data: the oracle's fp32 result rounded once, at most 1 ulp apart
+    a = ck.fill_uniform(dt, (M, K), 182, 0)
+    bt = ck.fill_uniform(dt, (N, K), 182, 1)
+    c16 = to16(ck.fill_uniform(ck.DT_F32, (M, N), 182, 2)) if with_c else None
+    got = run(a, bt, c16, policy).float().numpy()
+    ref = oracle.gemm(odt, a, bt, None if c16 is None else c16.float().numpy(), alpha, beta)
+    assert_close(oracle, ref, got)
+    ref16 = to16(ref).float().numpy()
+    assert np.all(np.abs(got - ref16) <= np.abs(ref16) * (2.0 ** -7 if is_bf else 2.0 ** -10) + 1e-3)
+
+
+@pytest.mark.parametrize("with_c", [False, True])
+def test_split_k_fp32_output_off_a_16_byte_boundary(ck, with_c):
+    # D (and C) four bytes into their allocations: the reduction pass takes its one-element-per-thread form
+    M, N, K = 512, 768, 8192
+    t = _straight_line_tuning(ck)
+    a = ck.fill_int(ck.DT_F16, (M, K), 183, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 183, 1, -2, 2)
+    c = ck.fill_int(ck.DT_F32, (M, N), 183, 2, -3, 3)
+    alpha, beta = (2.0, -1.0) if with_c else (1.0, 0.0)
+    want = alpha * (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float64)
+    if with_c:
+        want = want + beta * c
+    da, db = G.to_dev(a), G.to_dev(bt)
+    dbuf = torch.full((M * N + 8,), float("nan"), dtype=torch.float32, device="cuda")
+    cbuf = torch.zeros((M * N + 8,), dtype=torch.float32, device="cuda")
+    cbuf[1:1 + M * N] = torch.from_numpy(c.reshape(-1)).cuda()
+    for policy in (1, 4):
+        dbuf.fill_(float("nan"))
+        prev = ck.set_option(ck.OPT_SPLIT_K, policy)
+        try:
+            ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, da, db, cbuf.data_ptr() + 4 if with_c else None, dbuf.data_ptr() + 4, alpha, beta,
+                                            M, N, K, t["tile_dim"], t["segment_dim_k"], 0, 0, t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                            t["tile_group_m"], t["num_stages"], t["num_producer_warps"], t["num_consumer_warps"],
+                                            t["num_sms"])
+        finally:
+            ck.set_option(ck.OPT_SPLIT_K, prev)
+        assert ck.device_status() == 0
+        h = dbuf.cpu().numpy()
+        assert np.isnan(h[0]) and np.isnan(h[1 + M * N:]).all()          # nothing outside D is touched
+        assert np.array_equal(h[1:1 + M * N].reshape(M, N), want.astype(np.float32))
+
+
+# ---- 16384^3: the size the reference's own performance driver times (port_2.cu:1554-1556) -----------------------
+def test_16384_cubed_exact(ck):
+    M = N = K = 16384
+    t = suggested_tuning(ck, M, N, K)
+    # a one-hot Bt copies columns of A: every tile offset, every row and column position
+    a = ck.fill_int(ck.DT_F16, (M, K), 191, 0, -8, 8)
+    cols = (np.arange(N, dtype=np.int64) * 5 + 3) % K
+    eye = np.zeros((N, K), dtype=np.float16)
+    eye[np.arange(N), cols] = 1.0
+    d = G.run_gemm(ck, ck.DT_F16, a, eye, t=t)
+    assert np.array_equal(d, a[:, cols].astype(np.float32))
+    del eye
+    # small integers summed over the whole K: row and column sums of the exact product, and single rows
+    bt = ck.fill_int(ck.DT_F16, (N, K), 191, 1, -1, 1)
+    ai, bi = a.astype(np.int64), bt.astype(np.int64)      # |sum| <= 8 * 16384 < 2^24: exact in fp32
+    d = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+    assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
+    assert np.array_equal(d.astype(np.int64).sum(axis=0), bi @ ai.sum(axis=0))
+    for r in (0, 8191, 16383):
+        assert np.array_equal(d[r], (ai[r] @ bi.T).astype(np.float32))
+
+
+# ---- caller-owned workspace: the launcher allocates nothing -------------------------------------------------
+@pytest.mark.parametrize("name,dt_name,M,N,K", [
+    ("config 4", "f16", 2048, 2048, 32768),             # split-K planes: 4 x 16 MiB
+    ("config 5", "bf16", 6143, 4097, 3071),             # zero-padded operand copies: 60 MiB
+    ("copies and planes", "f16", 300, 520, 4090),       # both
+    ("16-bit C and D", "bf16", 512, 512, 8192),         # the <half, half> role through split-K
+])
+def test_workspace_entry_matches_the_allocating_launcher(ck, name, dt_name, M, N, K):
+    dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16
+    lp = name == "16-bit C and D"
+    t = suggested_tuning(ck, M, N, K)
+    order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b",
+                            "tile_group_m", "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
+    a = ck.fill_uniform(dt, (M, K), 201, 0)
+    bt = ck.fill_uniform(dt, (N, K), 201, 1)
+    da, db = G.to_dev(a), G.to_dev(bt)
+    tdt = torch.float32 if not lp else (torch.bfloat16 if dt == ck.DT_BF16 else torch.float16)
+    want = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+    (ck.gemm_shmem_tc_async_opt_port_lp if lp else ck.gemm_shmem_tc_async_opt_port)(dt, da, db, None, want, 1.0, 0.0, M, N, K, *order)
+    assert ck.device_status() == 0
+    need = ck.gemm_workspace_bytes(M, N, K, True, *order)
+    assert need > 0, "this launch is expected to need scratch memory"
+    ws = torch.empty(need + 64, dtype=torch.uint8, device="cuda")
+    got = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+    cd = dt if lp else ck.DT_F32
+    ck.gemm_shmem_tc_async_opt_port_ws(dt, cd, da, db, None, got, 1.0, 0.0, M, N, K, *order, ws.data_ptr() + 48, need)   # any alignment
+    assert ck.device_status() == 0
+    assert torch.equal(got.view(torch.int16 if lp else torch.int32), want.view(torch.int16 if lp else torch.int32))
+    # one byte short, or no workspace at all: an error before anything is written
+    for wptr, wbytes in ((ws.data_ptr() + 48, need - 257), (None, 0)):
+        got.fill_(7.0)
+        with pytest.raises(ck.CkoptError) as e:
+            ck.gemm_shmem_tc_async_opt_port_ws(dt, cd, da, db, None, got, 1.0, 0.0, M, N, K, *order, wptr, wbytes)
+        assert e.value.code == ck.ERR_TOO_LARGE
+        torch.cuda.synchronize()
+        assert float(got.float().min()) == float(got.float().max()) == 7.0
+
+
+def test_workspace_query_and_launches_that_need_none(ck):
+    # aligned operands, K a multiple of 8, enough tiles: no scratch, a NULL workspace is fine
+    M, N, K = 1024, 1024, 512
+    t = suggested_tuning(ck, M, N, K)
+    order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b",
+                            "tile_group_m", "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
+    assert ck.gemm_workspace_bytes(M, N, K, True, *order) == 0
+    assert ck.gemm_workspace_bytes(M, N, K, False, *order) >= (M + N) * K * 2      # unaligned operands are copied
+    assert ck.gemm_workspace_bytes(M, N, K - 3, True, *order) >= (M + N) * ((K - 3 + 7) // 8 * 8) * 2
+    a = ck.fill_int(ck.DT_F16, (M, K), 202, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 202, 1, -2, 2)
+    d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ck.gemm_shmem_tc_async_opt_port_ws(ck.DT_F16, ck.DT_F32, G.to_dev(a), G.to_dev(bt), None, d, 1.0, 0.0, M, N, K, *order, None, 0)
+    assert ck.device_status() == 0
+    assert np.array_equal(d.cpu().numpy(), (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32))
+    with pytest.raises(ck.CkoptError):
+        ck.gemm_workspace_bytes(M, N, K, True, 100, *order[1:])
