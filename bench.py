@@ -54,6 +54,24 @@ def load_package():
     return mod
 
 
+def mfma_ceiling(random_operands, with_loads, ksteps=400000):
+    """TFLOP/s the bare inner loop of the 256 x 256 tile GEMM sustains on the current device (no synchronisation, no
+    waiting for data, no epilogue): cuda-kernel-opt_amd/lib/libckmeasure.so, a measurement aid outside the product
+    library. int ckmeasure_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out)."""
+    import ctypes
+    path = os.path.join(ROOT, "cuda-kernel-opt_amd", "lib", "libckmeasure.so")
+    if not os.path.exists(path):
+        raise RuntimeError("libckmeasure.so is not built; run `python cuda-kernel-opt_amd/build.py`")
+    lib = ctypes.CDLL(path)
+    lib.ckmeasure_mfma_ceiling.restype = ctypes.c_int
+    lib.ckmeasure_mfma_ceiling.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    out = ctypes.c_double(0.0)
+    rc = lib.ckmeasure_mfma_ceiling(int(bool(random_operands)), int(bool(with_loads)), int(ksteps), ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError("ckmeasure_mfma_ceiling failed (%d)" % rc)
+    return out.value
+
+
 def cpu_baseline(ck, kind, dtype, a, b, M, N, K, budget_s=12.0):
     """Times the CPU oracle on a bounded row sample of the same operands; returns the JSON object."""
     from oracle import oracle as o
@@ -97,7 +115,9 @@ def sweep(ck, torch, args, ckdt, da, db, dd, M, N, K, cus, stream):
         wtr = ck.get_warp_tile_rows(tile, c)
         wave_rows = (wtr * 16, ck.get_num_acc(tile, c) // wtr * 16)
         for segk, stages, p in ((32, 5, 0), (32, 4, 0), (64, 2, 0), (128, 2, 0), (64, 2, 2), (64, 2, 4), (32, 4, 4), (64, 4, 2), (64, 4, 4), (128, 2, 2),
-                                 (64, 1, 2)):   # one stage: loads and MFMAs alternate, the no-pipeline partner
+                                 (64, 1, 2),    # one stage with producer waves: loads and MFMAs alternate
+                                 (64, 1, 0), (128, 1, 0)):   # one stage, no producers: the synchronous kernel (load, barrier, multiply,
+                                                             # barrier), the no-pipeline / no-specialisation partner of every other line
             tuples.append((tile, segk, 0, 0, tile, tile, args.group, stages, p, c))
         if tile >= 128:   # the finer synchronisation granularities of port_1 / port_2 (producer/consumer kernels only)
             tuples.append((tile, 64, 2, 1, wave_rows[0], wave_rows[1], args.group, 2 if tile == 256 else 4, 2, c))
@@ -168,7 +188,7 @@ def main():
                     help="run only a plain 1 GiB device copy kernel (reads 1 GiB, writes 1 GiB): the reference "
                          "reading for FETCH_SIZE / WRITE_SIZE counter runs")
     ap.add_argument("--ceiling", action="store_true",
-                    help="run only the bare inner-loop probe (ckopt_probe_mfma_ceiling): what the device sustains with "
+                    help="run only the bare inner-loop probe (libckmeasure.so): what the device sustains with "
                          "constant / random operands, without / with the direct-to-LDS loads")
     ap.add_argument("--no-ceiling", action="store_true", help="skip the bare inner-loop probe of the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -199,7 +219,7 @@ def main():
         for rnd in (0, 1):
             for loads in (0, 1):
                 key = "%s_operands_%s" % ("random" if rnd else "constant", "with_loads" if loads else "no_loads")
-                res[key] = round(ck.probe_mfma_ceiling(rnd, loads, 400000), 1)
+                res[key] = round(mfma_ceiling(rnd, loads, 400000), 1)
         print(json.dumps({"probe": "bare inner loop of the 256x256 tile GEMM, 8 waves per CU, ~0.2 s per case",
                           "unit": "TFLOP/s", "nominal_peak": PEAK_TFLOPS["mfma_f16"], **res}))
         return 0
@@ -389,7 +409,7 @@ def main():
         # what the bare inner loop of this tile shape sustains on this device with random operands and the
         # loads of the real data flow (no synchronisation, no waiting, no epilogue): the device's power limit
         # keeps it well below the nominal peak, and no kernel of this shape can exceed it
-        ceil = ck.probe_mfma_ceiling(1, 1, 400000)
+        ceil = mfma_ceiling(1, 1, 400000)
         out["roofline"]["measured_ceiling"] = round(ceil, 1)
         out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
     if check is not None:

@@ -61,10 +61,6 @@ _lib.ckopt_device_status.restype = _i
 _lib.ckopt_device_status.argtypes = [_p]
 _lib.ckopt_last_launch_clocks.restype = _i
 _lib.ckopt_last_launch_clocks.argtypes = [_p, ctypes.POINTER(_u64), ctypes.POINTER(_u64)]
-_lib.ckopt_probe_counters.restype = _i
-_lib.ckopt_probe_counters.argtypes = [_p, ctypes.POINTER(ctypes.c_uint), _i]
-_lib.ckopt_probe_mfma_ceiling.restype = _i
-_lib.ckopt_probe_mfma_ceiling.argtypes = [_i, _i, _i, ctypes.POINTER(ctypes.c_double)]
 _lib.ckopt_suggest_gemm_tuning.restype = _i
 _lib.ckopt_suggest_gemm_tuning.argtypes = [_i, _i, _i, _i, ctypes.POINTER(ctypes.c_int)]
 _lib.ckopt_set_option.restype = _i
@@ -86,9 +82,8 @@ EXPORTED_SYMBOLS = [
     "ckopt_gemm_shmem_tc_async_opt_port_1",
     "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
-    "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks", "ckopt_probe_counters",
+    "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks",
     "ckopt_suggest_gemm_tuning",
-    "ckopt_probe_mfma_ceiling",
     "ckopt_set_option", "ckopt_fill_uniform",
     "ckopt_fill_normal", "ckopt_fill_int", "ckopt_fill_constant", "ckopt_error_string",
 ]
@@ -266,21 +261,6 @@ def last_launch_clocks(stream=None):
     c, w = _u64(0), _u64(0)
     _check(_lib.ckopt_last_launch_clocks(_stream(stream), ctypes.byref(c), ctypes.byref(w)), "last_launch_clocks")
     return int(c.value), int(w.value)
-
-
-def probe_mfma_ceiling(random_operands, with_loads, ksteps=400000):
-    """TFLOP/s the bare GEMM inner loop sustains on the current device (see ckopt.h)."""
-    out = ctypes.c_double(0.0)
-    _check(_lib.ckopt_probe_mfma_ceiling(int(bool(random_operands)), int(bool(with_loads)), int(ksteps), ctypes.byref(out)),
-           "probe_mfma_ceiling")
-    return out.value
-
-
-def probe_counters(nwaves=16, stream=None):
-    """Per-wave counters of a measurement build (zeros otherwise): list of 8-word lists."""
-    buf = (ctypes.c_uint * (nwaves * 8))()
-    _check(_lib.ckopt_probe_counters(_stream(stream), buf, nwaves * 8), "probe_counters")
-    return [list(buf[w * 8:(w + 1) * 8]) for w in range(nwaves)]
 
 
 def suggest_gemm_tuning(M, N, K, num_cus=256):

@@ -1,8 +1,9 @@
 """Builds libckopt.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
 
 Usage: python build.py [--jobs N] [--force]
-Every translation unit is compiled to build/<name>.o (in parallel) and linked into lib/libckopt.so
-next to this file. hipcc cross-compiles gfx950 code objects without a GPU.
+Every translation unit under csrc/ is compiled to build/<name>.o (in parallel) and linked into lib/libckopt.so
+next to this file; measure/ (the bare inner-loop probe bench.py reports a ceiling from) becomes the separate
+lib/libckmeasure.so, which the product library does not contain. hipcc cross-compiles gfx950 code objects without a GPU.
 """
 import argparse
 import concurrent.futures
@@ -12,6 +13,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+MEASURE = os.path.join(HERE, "measure")
 BUILD = os.path.join(HERE, "build")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libckopt.so")
@@ -26,17 +28,17 @@ DEVICE_FLAGS = [
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-x", "c++"]
 
 
-def sources():
+def sources(root=CSRC):
     out = []
-    for name in sorted(os.listdir(CSRC)):
+    for name in sorted(os.listdir(root)):
         if name.endswith(".hip") or name.endswith(".cpp"):
-            out.append(os.path.join(CSRC, name))
+            out.append(os.path.join(root, name))
     return out
 
 
 def headers_mtime():
     m = 0.0
-    for root in (CSRC, os.path.join(HERE, "..", "include")):
+    for root in (CSRC, MEASURE, os.path.join(HERE, "..", "include")):
         for name in os.listdir(root):
             if name.endswith((".h", ".inc")):
                 m = max(m, os.path.getmtime(os.path.join(root, name)))
@@ -56,25 +58,27 @@ def compile_one(src, force, build_dir=None, extra=()):
 
 
 def build(jobs=8, force=False, verbose=True, out_dir=None, extra=()):
-    """out_dir/extra: build a variant (extra compiler flags, e.g. -DCK_PROBE_NO_MFMA) into another directory."""
+    """out_dir/extra: build a variant (extra compiler flags, e.g. a -D define) into another directory."""
     build_dir = os.path.join(out_dir, "build") if out_dir else BUILD
     lib_dir = out_dir if out_dir else LIBDIR
     lib = os.path.join(lib_dir, "libckopt.so")
     os.makedirs(build_dir, exist_ok=True)
     os.makedirs(lib_dir, exist_ok=True)
     srcs = sources()
-    objs = []
+    msrcs = sources(MEASURE)
+    objs, mobjs = [], []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        for obj, what in ex.map(lambda s: compile_one(s, force, build_dir, extra), srcs):
+        for src, (obj, what) in zip(srcs + msrcs, ex.map(lambda s: compile_one(s, force, build_dir, extra), srcs + msrcs)):
             if verbose:
                 print("[build] %-40s %s" % (os.path.basename(obj), what), flush=True)
-            objs.append(obj)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("link failed: %s\n%s\n%s" % (" ".join(cmd), r.stdout, r.stderr))
-    if verbose:
-        print("[build] linked %s" % lib, flush=True)
+            (mobjs if src in msrcs else objs).append(obj)
+    for target, members in ((lib, objs), (os.path.join(lib_dir, "libckmeasure.so"), mobjs)):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", target] + members
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed: %s\n%s\n%s" % (" ".join(cmd), r.stdout, r.stderr))
+        if verbose:
+            print("[build] linked %s" % target, flush=True)
     return lib
 
 

@@ -24,11 +24,13 @@ bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int
 constexpr int STREAM_K_MULTIPLE_HOST = 64;  // K extent of one loop body of the straight-line kernel
 hipError_t launch_gemm_fused_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_fused_bf16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
+hipError_t launch_gemm_sync_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
+hipError_t launch_gemm_sync_bf16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_matmul_shmem(int dtype, int tile, int accs, bool bt, dim3 grid, hipStream_t s, const SimtArgs& a);
 }  // namespace ck
 
 // One status word per device; the kernels OR a bit into it when a bounded flag wait gives up.
-__device__ unsigned int ck_status_word[8 + 16 * 8] = {};  // [8..]: per-wave cycle counters of measurement builds
+__device__ unsigned int ck_status_word[8] = {};  // [0]: status bits, [2..5]: cycles and reference ticks of the last launch
 
 // Scratch memory of the entry point that allocates nothing (ckopt_gemm_shmem_tc_async_opt_port_2_noalloc): the
 // zero-padded operand copies and the split-K planes of one launch. Every device the library runs on holds its own
@@ -366,6 +368,10 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             }
             if (!scratch_release(sc, ws, s) && e == hipSuccess) e = hipErrorUnknown;
         }
+    } else if (t.num_producer_waves == 0 && t.num_stages == 1) {
+        // one stage, no producers: load, barrier, multiply, barrier (the synchronous A/B partner)
+        e = dtype == CK_DT_F16 ? launch_gemm_sync_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a)
+                               : launch_gemm_sync_bf16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a);
     } else if (t.num_producer_waves == 0) {
         e = dtype == CK_DT_F16 ? launch_gemm_fused_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a)
                                : launch_gemm_fused_bf16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a);
@@ -588,19 +594,6 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
     if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
     *shader_cycles = (uint64_t)v[2] | ((uint64_t)v[3] << 32);
     *ref_ticks = (uint64_t)v[4] | ((uint64_t)v[5] << 32);
-    return ck::CK_OK;
-}
-
-int ckopt_probe_counters(void* stream, unsigned int* out, int nwords) {
-    unsigned int* p = nullptr;
-    const int rc = status_ptr_for_current_device(&p);
-    if (rc != ck::CK_OK) return rc;
-    if (!out) return ck::CK_ERR_NULL;
-    if (nwords < 0 || nwords > 16 * 8) return ck::CK_ERR_BAD_PARAM;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
-    if (hipMemcpyAsync(out, p + 8, sizeof(unsigned int) * nwords, hipMemcpyDeviceToHost, s) != hipSuccess) return ck::CK_ERR_HIP;
-    if (hipStreamSynchronize(s) != hipSuccess) return ck::CK_ERR_HIP;
     return ck::CK_OK;
 }
 

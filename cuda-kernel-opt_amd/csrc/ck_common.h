@@ -187,9 +187,10 @@ CK_HD int check_gemm_tuning(const GemmTuning& t) {
         if (t.bar_steps_a < 0 || t.bar_steps_a >= wtr) return CK_ERR_BAD_PARAM;
         if (t.bar_steps_b < 0 || t.bar_steps_b >= wtc) return CK_ERR_BAD_PARAM;
     }
-    // fused variant: the waves meet at the workgroup barrier once per segment (no finer granularity),
-    // and a stage is refilled while the next one is multiplied, so it needs at least two
-    if (t.num_producer_waves == 0 && (mode != CK_SYNC_TILE || t.num_stages < 2)) return CK_ERR_NO_INSTANCE;
+    // no producer waves: the waves meet at the workgroup barrier (no finer granularity). Two or more stages:
+    // the fused variant (a stage is refilled while the next one is multiplied); one stage: the synchronous
+    // load / barrier / multiply / barrier kernel
+    if (t.num_producer_waves == 0 && mode != CK_SYNC_TILE) return CK_ERR_NO_INSTANCE;
     // 64 accumulator blocks (256 registers) leave no room for a second wave on the SIMD
     if (get_num_acc(t.tile_dim, t.num_consumer_waves) > 32) return CK_ERR_NO_INSTANCE;
     if (t.num_producer_waves + t.num_consumer_waves > max_waves_for(t.tile_dim, t.num_consumer_waves)) return CK_ERR_NO_INSTANCE;

@@ -33,16 +33,6 @@
 
 #include "gemm_pc_kernel.hip.h"
 
-// columns of 16 x 16 blocks multiplied between the landing wait and the barrier
-#ifndef CK_FUSED_PRE_COLS
-#define CK_FUSED_PRE_COLS 1
-#endif
-
-// cache policy bits of the direct-to-LDS loads (tuning builds may set "nt", "sc0", "sc1")
-#ifndef CK_DMA_CPOL
-#define CK_DMA_CPOL ""
-#endif
-
 namespace ck {
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -50,10 +40,7 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 // 16 bytes per lane from a raw buffer straight into LDS at lds_dst + lane * 16. voff is range
 // checked against the descriptor (out of range lanes write zeros), soff is not.
 __device__ __forceinline__ void dma_load_b128(i32x4 rsrc, uint32_t lds_dst, uint32_t voff, uint32_t soff) {
-#if defined(CK_PROBE_NO_LOADS)  // measurement build only: nothing is loaded
-    return;
-#endif
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen " CK_DMA_CPOL " lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff)
                  : "memory");
@@ -68,11 +55,7 @@ __device__ __forceinline__ i32x4 make_rsrc(const void* base, uint32_t num_record
     return r;
 }
 // workgroup barrier that the compiler treats as a full memory clobber (no LDS access moves across)
-#if defined(CK_PROBE_NO_BARRIER)  // measurement build only (results are wrong without the barrier)
-__device__ __forceinline__ void wg_barrier() { asm volatile("" ::: "memory"); }
-#else
 __device__ __forceinline__ void wg_barrier() { asm volatile("s_barrier" ::: "memory"); }
-#endif
 __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 template <int N> __device__ __forceinline__ void use_fragment_array(const u32x4 (&f)[N]) {
@@ -103,7 +86,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
     constexpr int HALF = NI / CW > 0 ? NI / CW : 1;
     constexpr int VAR = CPR == 4 ? 1 : CPR == 8 ? 2 : 4;
     constexpr int LPK = LPW / KSTEPS;          // wave loads per wave and k-step
-    constexpr int PRE = CK_FUSED_PRE_COLS < WTC ? CK_FUSED_PRE_COLS : WTC - 1;
+    constexpr int PRE = 1;                     // columns of 16 x 16 blocks multiplied between the landing wait and the barrier
     static_assert(2 * NI % CW == 0 && LPW >= 1 && LPK * KSTEPS == LPW && LPK >= 1, "stage must split evenly over waves and k-steps");
 
     extern __shared__ __attribute__((aligned(1024))) char ck_smem[];
@@ -149,13 +132,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
     for (int ii = 0; ii < HALF; ++ii) goff_step[ii] = (uint32_t)(ii * CW) * load_step;
 
     auto open_tile = [&]() __attribute__((always_inline)) {
-#if defined(CK_PROBE_SAME_TILE)  // measurement build only: every workgroup loads the operands of tile (0, 0)
-        const TileRC rc{0, 0};
-#elif defined(CK_PROBE_SAME_ROW)  // measurement build only: every workgroup loads A of tile row 0
-        const TileRC rc{0, tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, l_tc).col};
-#else
         const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, l_tc);
-#endif
         const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE);
         const int ra = g.M - row_a < TILE ? g.M - row_a : TILE, rb = g.N - row_b < TILE ? g.N - row_b : TILE;
         nrec_a = (uint32_t)ra * pitch32;
@@ -235,11 +212,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         for (int i = 0; i < WTR; ++i) {
 #pragma unroll
             for (int j = 0; j < WTC; ++j) {
-#if defined(CK_PROBE_NO_EPILOGUE)  // measurement build only: nothing is written (except by a workgroup that never exists)
-                if (blockIdx.x == 0x7fffffff) epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
-#else
                 epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
-#endif
                 acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
@@ -249,13 +222,6 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
     // outstanding (a wave's loads complete in issue order; other memory operations in flight only
     // make the wait longer, never shorter)
     auto wait_landed = [&](int X) __attribute__((always_inline)) {
-#if defined(CK_PROBE_NO_LANDING_WAIT)  // measurement build only (results are wrong): loads are never waited for
-        return;
-#endif
-#if defined(CK_PROBE_WAIT0)  // measurement build only: always drain (what two stages need), no ladder
-        wait_vmcnt_imm<0>();
-        return;
-#endif
         const int later = issued_loads - (X + 1) * LPW;
         if (later == 2 * LPW) wait_vmcnt_imm<2 * LPW>();   // four stages in steady state
         else if (later == LPW) wait_vmcnt_imm<LPW>();      // three stages
@@ -264,19 +230,6 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         else wait_vmcnt_le((uint32_t)later);
     };
 
-#if defined(CK_PROBE_NO_MFMA)  // measurement build only: loads, waits and barriers without the multiplication
-#define CK_MFMA(b, a, c) (c)
-#else
-#define CK_MFMA(b, a, c) MfmaOp<DT>::run(b, a, c)
-#endif
-#if defined(CK_PROBE_TIMING)  // measurement build only: cycles in front of the LDS wait, the landing wait, the barrier
-    unsigned long long t_lds = 0, t_vm = 0, t_bar = 0;
-#define CK_T0() unsigned long long ck_t0 = clock64()
-#define CK_T1(acc) { const unsigned long long ck_t1 = clock64(); acc += ck_t1 - ck_t0; ck_t0 = ck_t1; }
-#else
-#define CK_T0()
-#define CK_T1(acc)
-#endif
     // One k-step. Its fragments are in f[P] (possibly still arriving); the next k-step's go to f[1-P].
     auto kstep = [&](auto parity, auto kstep_index) __attribute__((always_inline)) {
         constexpr int P = decltype(parity)::value;
@@ -295,29 +248,24 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
             // the previous segment were issued by the k-step before this one.)
             ld_mode = 0;
             if (has_next_seg && opened_segs < total_segs) open_segment();
-            CK_T0();
             // The last fragments of this segment must be in registers before the barrier releases
             // their stage. The wait is requested through a use of the registers the compiler can
             // see: behind a bare s_waitcnt in inline assembly it would still count these reads as
             // outstanding and pad every later fragment wait with the reads issued after the barrier.
             use_fragments(fa[P], fb[P]);
-            CK_T1(t_lds);
             if (has_next_seg) wait_landed(G + 1);
-            CK_T1(t_vm);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < PRE; ++j)
 #pragma unroll
-            for (int i = 0; i < WTR; ++i) acc[i][j] = CK_MFMA(fb[P][j], fa[P][i], acc[i][j]);
+            for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);
         // chunk of LPK loads this k-step issues: at a segment's last k-step (behind the barrier) chunk 0
         // of the segment that goes into the stage just released, otherwise the next chunk of the
         // segment opened at the previous segment's last k-step
         if (last_ks && has_next_seg) {
-            CK_T0();
             wg_barrier();
-            CK_T1(t_bar);
         }
         constexpr int CHUNK = last_ks ? 0 : KS + 1;
         __builtin_amdgcn_sched_barrier(0);
@@ -325,16 +273,8 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         // first, then Bt) and this k-step's loads, one every LSTRIDE columns
         constexpr int NF = WTR + WTC;                 // fragments to fetch
         constexpr int COLS = WTC - PRE;               // columns left to multiply
-#if defined(CK_FUSED_FETCH_PER)
-        constexpr int PER = CK_FUSED_FETCH_PER;       // fetches per column (tuning builds)
-#else
         constexpr int PER = (NF + COLS - 1) / COLS;   // fetches per column
-#endif
-#if defined(CK_FUSED_LOAD_STRIDE)
-        constexpr int LSTRIDE = CK_FUSED_LOAD_STRIDE;  // tuning builds
-#else
         constexpr int LSTRIDE = (COLS + LPK - 1) / LPK;
-#endif
 #pragma unroll
         for (int j = PRE; j < WTC; ++j) {
             // (after the very last k-step of the stream this fetches fragments nobody uses: the
@@ -342,10 +282,8 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
 #pragma unroll
             for (int q = 0; q < PER; ++q) {
                 const int f = (j - PRE) * PER + q;
-#if !defined(CK_PROBE_NO_MFMA)
                 if (f < WTR) fa[1 - P][f] = *(const CK_LDS u32x4*)(uintptr_t)(pa_k + f * 16 * RB);
                 else if (f < NF) fb[1 - P][f - WTR] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + (f - WTR) * 16 * RB);
-#endif
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -355,7 +293,7 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < WTR; ++i) acc[i][j] = CK_MFMA(fb[P][j], fa[P][i], acc[i][j]);
+            for (int i = 0; i < WTR; ++i) acc[i][j] = MfmaOp<DT>::run(fb[P][j], fa[P][i], acc[i][j]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -428,13 +366,6 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         }
     }
 
-#if defined(CK_PROBE_TIMING)
-    if (blockIdx.x == 0 && lane == 0) {
-        unsigned* o = g.status + 8 + wave * 8;
-        o[0] = (unsigned)t_vm; o[1] = (unsigned)(t_vm >> 32); o[2] = 0; o[3] = 0;
-        o[4] = (unsigned)(t_lds >> 4); o[5] = (unsigned)(t_vm >> 4); o[6] = (unsigned)(t_bar >> 4);
-    }
-#endif
     if (blockIdx.x == 0 && threadIdx.x == blockDim.x - 1) {
         const unsigned long long dc = clock64() - clk0, dw = wall_clock64() - wall0;
         g.status[2] = (unsigned)dc; g.status[3] = (unsigned)(dc >> 32);

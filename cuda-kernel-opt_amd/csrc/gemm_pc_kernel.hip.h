@@ -42,10 +42,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define CK_LDS __attribute__((address_space(3)))
 
-// Bt fragments kept resident per k-step when a wave tile has more than four block columns
-#ifndef CK_RESIDENT_BT_FRAGS
-#define CK_RESIDENT_BT_FRAGS 3
-#endif
+constexpr int RESIDENT_BT_FRAGS = 3;  // Bt fragments kept resident per k-step when a wave tile has more than four block columns
 
 struct GemmArgs {
     const void* A;
@@ -210,19 +207,11 @@ struct Spin {
     unsigned int* status;
     unsigned bit;
     bool dead;
-#if defined(CK_PROBE_TIMING)  // measurement build only: cycles spent and calls made in flag waits
-    unsigned long long wait_cycles = 0;
-    unsigned wait_calls = 0, wait_polls = 0;
-#endif
 };
 __device__ __forceinline__ bool flag_ready(uint32_t addr, uint32_t target) { return (int32_t)(flag_load(addr) - target) >= 0; }
 __device__ __forceinline__ void wait_flag_ge(uint32_t addr, uint32_t target, Spin& sp) {
     if (sp.dead) return;
     uint32_t n = 0;
-#if defined(CK_PROBE_TIMING)
-    const unsigned long long t0 = clock64();
-    struct Acc { Spin& s; unsigned long long t0; uint32_t& n; __device__ ~Acc() { s.wait_cycles += clock64() - t0; s.wait_calls++; s.wait_polls += n; } } acc_{sp, t0, n};
-#endif
     while (!flag_ready(addr, target)) {
         if (++n > sp.limit) {
             sp.dead = true;
@@ -284,10 +273,6 @@ template <int DEPTH>
 __device__ __forceinline__ void producer_wait(uint32_t addr, uint32_t target, SignalQueue<DEPTH>& q, Spin& sp, int nap) {
     if (target == 0 || sp.dead) return;
     uint32_t n = 0;
-#if defined(CK_PROBE_TIMING)
-    const unsigned long long t0 = clock64();
-    struct Acc { Spin& s; unsigned long long t0; uint32_t& n; __device__ ~Acc() { s.wait_cycles += clock64() - t0; s.wait_calls++; s.wait_polls += n; } } acc_{sp, t0, n};
-#endif
     while (!flag_ready(addr, target)) {
         if (q.pending()) {
             q.pop_front();
@@ -357,9 +342,6 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
     const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
     const int64_t total_tiles = (int64_t)g.tiles_m * g.tiles_n;
 
-#if defined(CK_PROBE_NO_SYNC)  // measurement build only: consumers run without any flag traffic
-    return;
-#endif
     Spin sp{g.spin_limit, g.status, CK_STATUS_PRODUCER_TIMEOUT, false};
     SignalQueue<MODE == CK_SYNC_TILE ? 3 : MODE == CK_SYNC_WAVE ? 4 : 8> sq;
     sq.init();
@@ -407,10 +389,6 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
                     if (sub <= s_own) producer_wait(fl + (empty_off + unit * (s_own + 1) + sub) * 4, readers * fill, sq, sp, g.producer_nap);
                 }
                 // ---- this wave's share of the row block, straight into LDS
-#if defined(CK_PROBE_NO_LOADS)  // measurement build only: producers signal without loading
-                if (true) {
-                } else
-#endif
                 if (fast) {
                     const uint32_t soff0 = (uint32_t)k0 * 2u;
 #pragma unroll
@@ -451,12 +429,6 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
         }
     }
     sq.drain();
-#if defined(CK_PROBE_TIMING)
-    if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
-        unsigned* o = g.status + 8 + (threadIdx.x >> 6) * 8;
-        o[0] = (unsigned)sp.wait_cycles; o[1] = (unsigned)(sp.wait_cycles >> 32); o[2] = sp.wait_calls; o[3] = sp.wait_polls;
-    }
-#endif
 }
 
 template <int TILE, int SEGK, int CW, int MODE, bool IS_A>
@@ -506,9 +478,6 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
     int stage = 0;
     uint32_t fill = 0;
     uint32_t pre_a = 0, pre_b = 0;  // "full" counters of the upcoming segment, read ahead of time
-#if defined(CK_PROBE_TIMING)
-    unsigned prefetch_hits = 0;
-#endif
     for (int64_t tc = slot; tc < total_tiles; tc += grid) {
         const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
         f32x4 acc[WTR][WTC];
@@ -525,14 +494,10 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
             if (MODE != CK_SYNC_ACC) {
                 // The two "full" counters of this segment were read one segment ahead (behind the
                 // previous segment's fragment reads); poll only if they were not there yet.
-#if !defined(CK_PROBE_NO_SYNC)
                 const uint32_t seen_a = __builtin_amdgcn_readfirstlane(pre_a);
                 const uint32_t seen_b = __builtin_amdgcn_readfirstlane(pre_b);
                 if ((int32_t)(seen_a - pa * (fill + 1)) < 0) wait_flag_ge(fullA + fa_idx * 4, pa * (fill + 1), sp);
                 if ((int32_t)(seen_b - pb * (fill + 1)) < 0) wait_flag_ge(fullB + fb_idx * 4, pb * (fill + 1), sp);
-#if defined(CK_PROBE_TIMING)
-                if ((int32_t)(seen_a - pa * (fill + 1)) >= 0 && (int32_t)(seen_b - pb * (fill + 1)) >= 0) prefetch_hits++;
-#endif
                 asm volatile("" ::: "memory");
                 {
                     const int nstage = stage + 1 == S ? 0 : stage + 1;
@@ -540,14 +505,13 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                     pre_a = flag_peek(nfl + fa_idx * 4);
                     pre_b = flag_peek(nfl + 2 * ua * 4 + fb_idx * 4);
                 }
-#endif
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) {
                     const uint32_t pa_k = (st + a_lane) ^ (uint32_t)(ks * 64), pb_k = (st + b_lane) ^ (uint32_t)(ks * 64);
                     // At most JB Bt fragments are resident; fragment j + JB replaces fragment j
                     // right after its last use, so a 4 x 8 wave tile needs 32 fragment registers
                     // next to its 128 accumulator registers.
-                    constexpr int JB = WTC > 4 ? CK_RESIDENT_BT_FRAGS : WTC;
+                    constexpr int JB = WTC > 4 ? RESIDENT_BT_FRAGS : WTC;
                     u32x4 a[WTR], b[JB];
                     // Fragment-load phase at low priority, MFMA burst at a raised one. The two consumer
                     // waves that share a SIMD raise to DIFFERENT levels: when both have MFMAs ready one
@@ -555,57 +519,34 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
                     // fragments while the other bursts, so the pair settles into ping-pong instead of
                     // stalling on LDS latency in lockstep.
                     if (g.prio_mode == 1) __builtin_amdgcn_s_setprio(0);
-#if defined(CK_PROBE_NO_LDS)  // measurement build only: fragments are made up in registers
-#pragma unroll
-                    for (int i = 0; i < WTR; ++i) a[i] = u32x4{pa_k, pa_k + i, 1u, 2u};
-#pragma unroll
-                    for (int j = 0; j < JB; ++j) b[j] = u32x4{pb_k, pb_k + j, 3u, 4u};
-#else
 #pragma unroll
                     for (int i = 0; i < WTR; ++i) a[i] = *(const CK_LDS u32x4*)(uintptr_t)(pa_k + i * 16 * RB);
 #pragma unroll
                     for (int j = 0; j < JB; ++j) b[j] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + j * 16 * RB);
-#endif
                     __builtin_amdgcn_sched_barrier(0);
                     if (g.prio_mode == 1) {
                         if (burst_hi) __builtin_amdgcn_s_setprio(2);
                         else __builtin_amdgcn_s_setprio(1);
                     }
                     __builtin_amdgcn_sched_barrier(0);
-#if !defined(CK_PROBE_NO_SYNC)
                     if (ks == KSTEPS - 1 && JB == WTC) {
                         flag_add_after_reads(emptyA + fa_idx * 4);
                         flag_add(emptyB + fb_idx * 4);
                     }
-#endif
 #pragma unroll
                     for (int j = 0; j < WTC; ++j) {
-#if !defined(CK_PROBE_NO_SYNC)
                         if (ks == KSTEPS - 1 && JB != WTC && j == WTC - 1) {
                             flag_add_after_reads(emptyA + fa_idx * 4);
                             flag_add(emptyB + fb_idx * 4);
                         }
-#endif
 #pragma unroll
                         for (int i = 0; i < WTR; ++i) {
-#if defined(CK_PROBE_NO_MFMA)  // measurement build only: consumers read fragments but skip the MFMAs
-                            asm volatile("" ::"v"(b[j % JB]), "v"(a[i]));
-#else
                             acc[i][j] = MfmaOp<DT>::run(b[j % JB], a[i], acc[i][j]);
-#endif
                         }
                         if (j + JB < WTC) {
-#if !defined(CK_PROBE_NO_SCHED_BARRIER)
                             __builtin_amdgcn_sched_barrier(0);
-#endif
-#if defined(CK_PROBE_NO_LDS)
-                            b[j % JB] = u32x4{pb_k, pb_k + j, 5u, 6u};
-#else
                             b[j % JB] = *(const CK_LDS u32x4*)(uintptr_t)(pb_k + (j + JB) * 16 * RB);
-#endif
-#if !defined(CK_PROBE_NO_SCHED_BARRIER)
                             __builtin_amdgcn_sched_barrier(0);
-#endif
                         }
                     }
                 }
@@ -665,13 +606,6 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
             if (++stage == S) { stage = 0; ++fill; }
         }
 
-#if defined(CK_PROBE_TIMING)
-        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) {
-            unsigned* o = g.status + 8 + (threadIdx.x >> 6) * 8;
-            o[0] = (unsigned)sp.wait_cycles; o[1] = (unsigned)(sp.wait_cycles >> 32); o[2] = sp.wait_calls; o[3] = sp.wait_polls;
-            o[4] = prefetch_hits;
-        }
-#endif
         // ---- epilogue: D = alpha * acc + beta * C straight from the accumulators. With the Bt
         // fragment as the first MFMA operand a lane holds 4 consecutive columns of one row.
         const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);

@@ -143,7 +143,7 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_pcb_kernel(const GemmArgs g) {
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) {
                     const uint32_t pa_k = (st + a_lane) ^ (uint32_t)(ks * 64), pb_k = (st + b_lane) ^ (uint32_t)(ks * 64);
-                    constexpr int JB = WTC > 4 ? CK_RESIDENT_BT_FRAGS : WTC;
+                    constexpr int JB = WTC > 4 ? RESIDENT_BT_FRAGS : WTC;
                     u32x4 a[WTR], b[JB];
 #pragma unroll
                     for (int i = 0; i < WTR; ++i) a[i] = *(const CK_LDS u32x4*)(uintptr_t)(pa_k + i * 16 * RB);

@@ -41,15 +41,6 @@
 
 #include "gemm_fused_kernel.hip.h"
 
-// schedule constants (tuning builds override them)
-#ifndef CK_STREAM_PRE
-#define CK_STREAM_PRE 1
-#endif
-#ifndef CK_STREAM_LOAD_COL_0
-#define CK_STREAM_LOAD_COL_0 3
-#define CK_STREAM_LOAD_COL_1 6
-#endif
-
 namespace ck {
 
 constexpr int STREAM_TILE = 256;
@@ -66,12 +57,20 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     constexpr int OPB = TILE * RB;           // one operand's part of a quarter
     constexpr int QB = 2 * OPB;              // one quarter
     constexpr int LPB = 8;                   // loads per wave and body: (A, Bt) x (rows w, w + 8) x (two halves)
-    constexpr int EPILOGUE_STORES = WTR * WTC;
-    constexpr int PRE = CK_STREAM_PRE;               // columns of MFMAs in front of the barrier
-    constexpr int LOAD_COL_0 = CK_STREAM_LOAD_COL_0;  // columns behind which a k-step's two load pairs are issued
-    constexpr int LOAD_COL_1 = CK_STREAM_LOAD_COL_1;
+    // Stores one wave issues in the epilogue of an interior tile. The landing wait of the body behind an epilogue
+    // counts them (they sit between the loads in flight and the new ones), so the loops below and the wait
+    // immediates are written in terms of the same constants.
+    constexpr int F32_GROUP = 2, H16_GROUP = 4;     // accumulator blocks exchanged between lanes into whole lines
+    constexpr int STORES_PER_GROUP = 2;             // rows 0..7 and 8..15 of the group
+    constexpr int EPILOGUE_STORES = WTR * (WTC / F32_GROUP) * STORES_PER_GROUP;        // fp32 output
+    constexpr int EPILOGUE_STORES_16 = WTR * (WTC / H16_GROUP) * STORES_PER_GROUP;     // 16-bit output
+    static_assert(WTC % F32_GROUP == 0 && WTC % H16_GROUP == 0, "whole groups per wave-tile row");
+    static_assert(EPILOGUE_STORES_16 * 2 == EPILOGUE_STORES, "count_stores selects between the two with a shift by one");
+    constexpr int PRE = 1;               // columns of MFMAs in front of the barrier
+    constexpr int LOAD_COL_0 = 3;  // columns behind which a k-step's two load pairs are issued
+    constexpr int LOAD_COL_1 = 6;
     static_assert(PRE >= 1 && (WTC - PRE) * 2 >= WTR + WTC && LOAD_COL_0 >= PRE && LOAD_COL_1 > LOAD_COL_0 && LOAD_COL_1 < WTC, "schedule");
-    static_assert(LPB + EPILOGUE_STORES < 64, "the wait immediates must fit the 6-bit counter");
+    static_assert(LPB + EPILOGUE_STORES < 64 && EPILOGUE_STORES_16 < EPILOGUE_STORES, "the wait immediates must fit the 6-bit counter");
     static_assert(STREAM_LDS_BYTES <= LDS_BYTES_PER_CU, "the ring is all of the LDS");
 
     extern __shared__ __attribute__((aligned(1024))) char ck_smem[];
@@ -119,11 +118,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         if (l_tile < my_tiles) {
             int slice = 0;
             const int64_t tc = item_tile(slot + (int64_t)l_tile * grid, slice);
-#if defined(CK_PROBE_SAME_TILE)  // measurement build only: every workgroup loads the operands of tile (0, 0)
-            const TileRC rc{0, 0};
-#else
             const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
-#endif
             const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE);
             const int ra = g.M - row_a < TILE ? g.M - row_a : TILE, rb = g.N - row_b < TILE ? g.N - row_b : TILE;
             const int64_t k0 = (int64_t)slice * kslice_bytes;  // the slice starts k0 bytes into every row
@@ -182,9 +177,6 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                  : "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(uint32_t, g.beta))),
                    "s"(__builtin_amdgcn_readfirstlane((uint32_t)g.out16)), "s"(__builtin_amdgcn_readfirstlane(d16_misaligned))
                  : "scc");
-#if defined(CK_PROBE_TIMING)  // measurement build only: cycles in the epilogues, in the first and second loop body behind one, in all others
-    unsigned long long t_epi = 0, t_first = 0, t_second = 0, t_other = 0;
-#endif
     uint32_t stores_in_flight;  // nonzero in the loop body that follows an epilogue whose stores count in the wait
     asm volatile("s_mov_b32 %0, 0" : "=s"(stores_in_flight));
     // byte offsets in the ring of the quarters of the even k-step (q0) and of the four after it
@@ -195,7 +187,6 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     auto kstep = [&](auto parity, uint32_t qn) __attribute__((always_inline)) {
         constexpr int P = decltype(parity)::value;
         use_fragments(fa[P], fb[P]);
-#if !defined(CK_PROBE_NO_LANDING_WAIT)  // measurement builds drop the wait (results are wrong)
         if constexpr (P == 1) {
             // loads of the next two k-steps landed: after them this wave issued the four loads of
             // this body's even k-step and, behind an epilogue, the epilogue's stores. (The choice
@@ -205,11 +196,10 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             asm volatile("s_cmp_lg_u32 %0, 0\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(%1)\n1:\n\t"
                          "s_cmp_eq_u32 %0, 2\n\ts_cbranch_scc1 2f\n\ts_waitcnt vmcnt(%2)\n2:\n\ts_waitcnt vmcnt(%3)"
                          :
-                         : "s"(stores_in_flight), "n"(ODD_ONLY ? 0 : LPB / 2), "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES / 2),
+                         : "s"(stores_in_flight), "n"(ODD_ONLY ? 0 : LPB / 2), "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES_16),
                            "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES)
                          : "memory", "scc");
         }
-#endif
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < PRE; ++j)
@@ -281,9 +271,6 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 
         for (int t = 0; t < my_tiles; ++t) {
             for (int b = 0; b < nb; ++b) {
-#if defined(CK_PROBE_TIMING)
-                const unsigned long long tb0 = clock64();
-#endif
                 kstep(std::integral_constant<int, 0>{}, q1);
                 kstep(std::integral_constant<int, 1>{}, q2);
                 loader_advance();
@@ -295,13 +282,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                     if (n1 == (uint32_t)(NQ * QB)) n1 = 0;
                     q0 = n0; q1 = n1; q2 = n2; q4 = n4;
                 }
-#if defined(CK_PROBE_TIMING)
-                { const unsigned long long d = clock64() - tb0; if (b == 0 && t > 0) t_first += d; else if (b == 1 && t > 0) t_second += d; else t_other += d; }
-#endif
             }
-#if defined(CK_PROBE_TIMING)
-            const unsigned long long te0 = clock64();
-#endif
             // D = alpha * acc + beta * C straight from the accumulators
             int slice = 0;
             const int64_t tc = item_tile(slot + (int64_t)t * grid, slice);
@@ -311,14 +292,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
             const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
             const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
-#if defined(CK_PROBE_NO_EPILOGUE)  // measurement build only: nothing is written (except by a workgroup that never exists)
-            if (blockIdx.x == 0x7fffffff)
-#endif
-#if defined(CK_STREAM_BLOCK_STORES)  // tuning builds: one store per accumulator block (half lines)
-            if (false) {
-#else
             if (interior && !g.out16) {
-#endif
                 // Whole 128-byte lines per store: an accumulator block gives a row 64 bytes (4 lanes x 16),
                 // and the write path's cost is per request, not per byte. Two neighbouring blocks are
                 // exchanged between lanes so that 8 lanes hold the 32 consecutive floats of one row:
@@ -333,9 +307,9 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
                 for (int i = 0; i < WTR; ++i) {
 #pragma unroll
-                    for (int j = 0; j < WTC; j += 2) {
+                    for (int j = 0; j < WTC; j += F32_GROUP) {
 #pragma unroll
-                        for (int tt = 0; tt < 2; ++tt) {
+                        for (int tt = 0; tt < STORES_PER_GROUP; ++tt) {
                             f32x4 v;
 #pragma unroll
                             for (int e = 0; e < 4; ++e) {
@@ -378,7 +352,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
                 for (int i = 0; i < WTR; ++i) {
 #pragma unroll
-                    for (int j = 0; j < WTC; j += 4) {
+                    for (int j = 0; j < WTC; j += H16_GROUP) {
                         const u32x4 first = packed_pair(acc[i][j], acc[i][j + 1]);
                         const u32x4 second = packed_pair(acc[i][j + 2], acc[i][j + 3]);
                         u32x4 other;  // the second pair's piece of the row 8 away
@@ -386,7 +360,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                         for (int e = 0; e < 4; ++e)
                             other[e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)second[e], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
 #pragma unroll
-                        for (int tt = 0; tt < 2; ++tt) {
+                        for (int tt = 0; tt < STORES_PER_GROUP; ++tt) {
                             const bool own = low_rows == (tt == 0);  // this lane's row is among the store's 8 rows
                             u32x4 o;
 #pragma unroll
@@ -406,9 +380,6 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             for (int i = 0; i < WTR; ++i)
 #pragma unroll
                 for (int j = 0; j < WTC; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-#if defined(CK_PROBE_TIMING)
-            t_epi += clock64() - te0;
-#endif
             // (set through asm so that the flag stays one opaque scalar register: otherwise the compiler
             // peels the loop around its known values)
             asm volatile("s_mov_b32 %0, %1" : "=s"(stores_in_flight) : "s"(interior ? count_stores : 0u));
@@ -417,12 +388,6 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         wait_vmcnt_imm<0>();
     }
 
-#if defined(CK_PROBE_TIMING)
-    if (blockIdx.x == 0 && lane == 0) {
-        unsigned* o = g.status + 8 + wave * 8;
-        o[0] = (unsigned)(t_epi >> 4); o[1] = (unsigned)(t_first >> 4); o[2] = (unsigned)(t_second >> 4); o[3] = (unsigned)(t_other >> 4);
-    }
-#endif
     if (blockIdx.x == 0 && threadIdx.x == blockDim.x - 1) {
         const unsigned long long dc = clock64() - clk0, dw = wall_clock64() - wall0;
         g.status[2] = (unsigned)dc; g.status[3] = (unsigned)(dc >> 32);

@@ -183,17 +183,13 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
         }
     };
 
-    // CK_PROBE_SIMT_NOSTASH / CK_PROBE_SIMT_NOLDS: measurement builds only (wrong results): the loop without
-    // the global loads and LDS writes of the next slice / with one LDS read per slice instead of one per k.
     fetch(0);
     stash(0);
     __syncthreads();
     int buf = 0;
     for (int k0 = 0; k0 < K; k0 += KT) {
         const bool more = k0 + KT < K;
-#ifndef CK_PROBE_SIMT_NOSTASH
         if (more) fetch(k0 + KT);
-#endif
         if (ROT) {
 #pragma unroll
             for (int i = 0; i < RM; ++i)
@@ -202,32 +198,19 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
         }
         const ACC* as = a_s(buf) + ty * RM;
         const ACC* bs = b_s(buf) + tx * RN;
-#ifdef CK_PROBE_SIMT_NOLDS
-        ACC av[RM], bv[RN];
-#pragma unroll
-        for (int i = 0; i < RM; ++i) av[i] = as[i];
-#pragma unroll
-        for (int j = 0; j < RN; ++j) bv[j] = bs[j];
-#endif
 #pragma unroll(K_UNROLL)
         for (int k = 0; k < KT; ++k) {
-#ifndef CK_PROBE_SIMT_NOLDS
             ACC av[RM], bv[RN];
 #pragma unroll
             for (int i = 0; i < RM; ++i) av[i] = as[k * LD + i];
 #pragma unroll
             for (int j = 0; j < RN; ++j) bv[j] = bs[k * LD + j];
-#else
-            asm volatile("" ::: "memory");
-#endif
 #pragma unroll
             for (int i = 0; i < RM; ++i)
 #pragma unroll
                 for (int j = 0; j < RN; ++j) acc_set(i, j, SimtIo<DT>::mad(av[i], bv[j], acc_get(i, j)));
         }
-#ifndef CK_PROBE_SIMT_NOSTASH
         if (more) stash(buf ^ 1);
-#endif
         __syncthreads();
         buf ^= 1;
     }

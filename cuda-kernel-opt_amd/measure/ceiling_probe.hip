@@ -10,7 +10,7 @@
 
 #include <stdint.h>
 
-#include "ck_common.h"
+#include "../csrc/ck_common.h"
 
 namespace {
 
@@ -116,7 +116,11 @@ hipError_t launch_probe(int cus, const char* window, int ksteps, float* sink, hi
 
 }  // namespace
 
-extern "C" int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out) {
+// Built into lib/libckmeasure.so, a measurement aid that bench.py loads next to the product library (which does not
+// contain it). random_operands: random instead of constant fragment values; with_loads: also the direct-to-LDS loads;
+// runs ksteps k-steps per wave on every CU after a warm-up, allocates and frees its own buffers, synchronises, and
+// returns the rate in TFLOP/s.
+extern "C" int ckmeasure_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out) {
     using namespace ck;
     if (!tflops_out || ksteps < 2 || ksteps > (1 << 26)) return CK_ERR_BAD_PARAM;
     int dev = 0, cus = 0;

@@ -49,7 +49,8 @@ enum {
  * with bar_steps_a < wave_tile_rows and bar_steps_b < wave_tile_cols; num_producer_waves in
  * {2,4,8} (half stream A, half stream Bt) or 0 (no dedicated producers: every consumer wave also
  * streams its share of each segment and the waves meet at the workgroup barrier once per segment;
- * tile granularity only, num_stages >= 2); num_consumer_waves in {4,8}; num_cus = persistent grid.
+ * tile granularity only; with num_stages 1 nothing overlaps: load, barrier, multiply, barrier, the schedule of the
+ * reference's first tensor-core kernel, matmul_shmem_tc.cu:105-231); num_consumer_waves in {4,8}; num_cus = persistent grid.
  * M, N need not be multiples of tile_dim and K need not be a multiple of segment_dim_k (edges are
  * zero-filled / masked). The kernels read operand rows that start on 16-byte boundaries: when K is
  * not a multiple of 8, or A / Bt is not 16-byte aligned (2-byte alignment is required), the call
@@ -171,22 +172,6 @@ int ckopt_device_status(void* stream);
  * the compute units actually ran at (it drops under matrix-core load), which turns a duration into a
  * matrix-core utilisation. No reference counterpart. */
 int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* ref_ticks);
-
-/* Copies up to 128 words of per-wave cycle counters that measurement builds of the library
- * (compiled with -DCK_PROBE_TIMING) record for workgroup 0: 8 words per wave - cycles spent in
- * flag waits (lo, hi), wait calls, polls, read-ahead hits. All zero in the normal build. */
-int ckopt_probe_counters(void* stream, unsigned int* out, int nwords);
-
-/* Measures what the inner loop of the 256 x 256 tile GEMM sustains on the current device when nothing
- * of a real GEMM is in its way (no synchronisation, no waiting for data, no epilogue): 8 waves per CU,
- * per wave and k-step 32 MFMAs on fragments read from LDS one k-step ahead, with with_loads != 0 also
- * the four direct-to-LDS loads per wave and k-step of the real data flow (from an L2-resident
- * window). random_operands selects random instead of constant fragment values: the power the matrix
- * cores draw, and with it the clock the device sustains, depends on the operand values. Runs ksteps
- * k-steps per wave on every CU (after a warm-up), allocates and frees its own buffers, synchronises,
- * and returns the rate in TFLOP/s: the practical ceiling next to the nominal peak. No reference
- * counterpart. */
-int ckopt_probe_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out);
 
 /* Process-wide tuning switches that are not launcher parameters in the reference:
  * key 0: LDS XOR swizzle on/off (default 1); key 1: spin limit of bounded waits (default 1<<22);

@@ -103,30 +103,44 @@ static int correctness(int cus) {
     return failed;
 }
 
-// uniform[-1,1) operands; number of elements with |cpu - gpu| > 0.1 (the reference's accuracy count) must be 0
-static int accuracy(int cus) {
-    const int dim = 512;
-    const size_t n = (size_t)dim * dim;
-    std::vector<DT> a(n), b(n);
-    std::vector<DT_ACC> c(n), res(n), ref(n);
-    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F16, a.data(), (int64_t)n, 77, 0, -1.f, 1.f), "fill");
-    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F16, b.data(), (int64_t)n, 77, 1, -1.f, 1.f), "fill");
-    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F32, c.data(), (int64_t)n, 77, 2, -1.f, 1.f), "fill");
-    if (oracle_gemm_blocked(0, (const uint16_t*)a.data(), (const uint16_t*)b.data(), c.data(), ref.data(), 1.f, 1.f, dim, dim, dim, 0, dim, 0) != 0) return 1;
-    Device d(n);
-    HIP_OK(hipMemcpy(d.A, a.data(), n * sizeof(DT), hipMemcpyHostToDevice));
-    HIP_OK(hipMemcpy(d.B, b.data(), n * sizeof(DT), hipMemcpyHostToDevice));
-    HIP_OK(hipMemcpy(d.C, c.data(), n * sizeof(DT_ACC), hipMemcpyHostToDevice));
+// uniform[-1,1) operands; number of elements with |cpu - gpu| > 0.1 (the reference's accuracy count) must be 0.
+// T is the element type (fp16 or bf16); M, N, K need not be multiples of anything.
+template <typename T>
+static int accuracy_shape(int M, int N, int K, int stride, int cus) {
+    const int dtype = ckopt::dtype_of<T>::value;
+    std::vector<T> a((size_t)M * K), b((size_t)N * K);
+    std::vector<DT_ACC> c((size_t)M * N), res((size_t)M * N), ref((size_t)M * N);
+    ckopt::check(ckopt_fill_uniform(dtype, a.data(), (int64_t)a.size(), 77, 0, -1.f, 1.f), "fill");
+    ckopt::check(ckopt_fill_uniform(dtype, b.data(), (int64_t)b.size(), 77, 1, -1.f, 1.f), "fill");
+    ckopt::check(ckopt_fill_uniform(CKOPT_DT_F32, c.data(), (int64_t)c.size(), 77, 2, -1.f, 1.f), "fill");
+    if (oracle_gemm_blocked(dtype, (const uint16_t*)a.data(), (const uint16_t*)b.data(), c.data(), ref.data(), 1.f, 1.f, M, N, K, 0, M, 0) != 0) return 1;
+    T *dA = nullptr, *dB = nullptr;
+    DT_ACC *dC = nullptr, *dD = nullptr;
+    HIP_OK(hipMalloc((void**)&dA, a.size() * sizeof(T))); HIP_OK(hipMalloc((void**)&dB, b.size() * sizeof(T)));
+    HIP_OK(hipMalloc((void**)&dC, c.size() * sizeof(DT_ACC))); HIP_OK(hipMalloc((void**)&dD, c.size() * sizeof(DT_ACC)));
+    HIP_OK(hipMemcpy(dA, a.data(), a.size() * sizeof(T), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dB, b.data(), b.size() * sizeof(T), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dC, c.data(), c.size() * sizeof(DT_ACC), hipMemcpyHostToDevice));
     int failed = 0, run = 0;
-    for (const Tuple& t : tuples(23)) {
-        HIP_OK(hipMemset(d.D, 0, n * sizeof(DT_ACC)));
-        launch(d, 1.f, 1.f, dim, t, cus);
-        HIP_OK(hipMemcpy(res.data(), d.D, n * sizeof(DT_ACC), hipMemcpyDeviceToHost));
-        const long long bad = (long long)oracle_count_incorrect(ref.data(), res.data(), (int64_t)n, 0.1f);
+    for (const Tuple& t : tuples(stride)) {
+        HIP_OK(hipMemset(dD, 0, c.size() * sizeof(DT_ACC)));
+        ckopt::gemm_shmem_tc_async_opt_port<T, DT_ACC>(dA, dB, dC, dD, 1.f, 1.f, M, N, K, t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b,
+                                                      t.rows_a, t.rows_b, t.tile_group_m, t.num_stages, t.producers, t.consumers, cus);
+        HIP_OK(hipMemcpy(res.data(), dD, c.size() * sizeof(DT_ACC), hipMemcpyDeviceToHost));
+        const long long bad = (long long)oracle_count_incorrect(ref.data(), res.data(), (int64_t)c.size(), 0.1f);
         ++run;
         if (bad != 0 || ckopt_device_status(nullptr) != 0) { ++failed; print_tuple(t); std::printf(": %lld incorrect\n", bad); }
     }
-    std::printf("accuracy: %d tuples at %d^3, %d with incorrect elements\n", run, dim, failed);
+    (void)hipFree(dA); (void)hipFree(dB); (void)hipFree(dC); (void)hipFree(dD);
+    std::printf("accuracy: %s %d x %d x %d, %d tuples, %d with incorrect elements\n", dtype == CKOPT_DT_F16 ? "fp16" : "bf16", M, N, K, run, failed);
+    return failed;
+}
+
+static int accuracy(int cus) {
+    int failed = accuracy_shape<ckopt::half_t>(512, 512, 512, 23, cus);        // the reference's own accuracy size
+    failed += accuracy_shape<ckopt::bfloat16_t>(512, 512, 512, 41, cus);
+    failed += accuracy_shape<ckopt::half_t>(500, 392, 520, 41, cus);           // ragged in every dimension, K not a multiple of 64
+    failed += accuracy_shape<ckopt::bfloat16_t>(333, 257, 1001, 67, cus);      // rows off 16-byte boundaries: zero-padded copies
     return failed;
 }
 

@@ -243,6 +243,33 @@ def test_fused_variant_no_producer_waves(ck, oracle, tile, c):
     assert_close(oracle, ref, G.run_gemm(ck, ck.DT_BF16, a2, b2, c2, 1.5, -0.5, t=make_tuning(ck, tile, 32, 4, 0, c)))
 
 
+@pytest.mark.parametrize("dt_name", ["f16", "bf16"])
+def test_synchronous_single_stage_partner(ck, oracle, dt_name):
+    # num_producer_waves 0 with ONE stage: load, barrier, multiply, barrier (the schedule of the reference's first
+    # tensor-core kernel, matmul_shmem_tc.cu:176-209), every tile size / segment size / wave count it is built for
+    dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16
+    odt = oracle.DT_F16 if dt_name == "f16" else oracle.DT_BF16
+    is_bf = dt_name == "bf16"
+    M, N, K = 300, 520, 328          # ragged in M and N; K ends inside a segment for every segment size
+    a = ck.fill_int(dt, (M, K), 53, 0, -2, 2)
+    bt = ck.fill_int(dt, (N, K), 53, 1, -2, 2)
+    c = ck.fill_int(ck.DT_F32, (M, N), 53, 2, -3, 3)
+    want = (2.0 * (G.as_f64(is_bf, a) @ G.as_f64(is_bf, bt).T) - c).astype(np.float32)
+    au = ck.fill_uniform(dt, (512, 1024), 54, 0)
+    bu = ck.fill_uniform(dt, (768, 1024), 54, 1)
+    ref = oracle.gemm(odt, au, bu)
+    n = 0
+    for tile, cw in ((64, 4), (64, 8), (128, 4), (128, 8), (256, 8)):
+        for sk in (32, 64, 128):
+            t = make_tuning(ck, tile, sk, 1, 0, cw, group=3, cus=7)
+            assert legal(ck, t), t
+            assert np.array_equal(G.run_gemm(ck, dt, a, bt, c, 2.0, -1.0, t=t), want), t
+            t["num_sms"] = 256
+            assert_close(oracle, ref, G.run_gemm(ck, dt, au, bu, t=t))
+            n += 1
+    assert n == 15
+
+
 def test_port_0_and_port_1_entry_points(ck):
     M, N, K = 256, 384, 512
     a = ck.fill_int(ck.DT_F16, (M, K), 41, 0, -2, 2)
@@ -393,11 +420,12 @@ def test_fused_variant_full_size(ck, oracle):
 
 
 def test_inner_loop_ceiling_probe_runs(ck):
-    # measurement helper: finite positive rates, and the loads never make the bare loop faster
-    r = {(rnd, ld): ck.probe_mfma_ceiling(rnd, ld, 20000) for rnd in (0, 1) for ld in (0, 1)}
+    # measurement aid of bench.py (libckmeasure.so, outside the product library): finite positive rates
+    import bench
+    r = {(rnd, ld): bench.mfma_ceiling(rnd, ld, 20000) for rnd in (0, 1) for ld in (0, 1)}
     assert all(np.isfinite(v) and 50.0 < v < 2600.0 for v in r.values()), r
-    with pytest.raises(ck.CkoptError):
-        ck.probe_mfma_ceiling(0, 0, 1)
+    with pytest.raises(RuntimeError):
+        bench.mfma_ceiling(0, 0, 1)
 
 
 def test_cpp_driver_through_the_launcher_templates(ck):

@@ -85,6 +85,7 @@ def test_tuning_legality_mirrors_reference_asserts(ck):
     assert ok(num_producer_waves=3) == ck.ERR_BAD_PARAM                                      # :1122
     assert ok(num_producer_waves=0) == ck.OK                 # fused variant (extension), tile granularity only
     assert ok(num_producer_waves=0, bar_step_rows_a=64, bar_step_rows_b=64) == ck.ERR_NO_INSTANCE
+    assert ok(num_producer_waves=0, num_stages=1) == ck.OK   # one stage: the synchronous load / barrier / multiply / barrier kernel
     assert ok(num_consumer_waves=6) == ck.ERR_BAD_PARAM                                      # :1123
     assert ok(num_stages=0) == ck.ERR_BAD_PARAM                                              # :1121
     assert ok(tile_group_m=0) == ck.ERR_BAD_PARAM

@@ -86,3 +86,21 @@ def test_config2_fp32_4096_b_transposed(ck, oracle, block_rows):
     rhs = a.astype(np.float64) @ b.astype(np.float64).sum(axis=0)
     scale = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).sum(axis=0) + 1.0
     assert np.max(np.abs(lhs - rhs) / scale) < 1e-5
+
+
+def test_cpp_driver_through_the_matmul_shmem_template(ck):
+    # the C++ face (ckopt::matmul_shmem<DT, DT_ACC>) driven by a test main in the role of the reference's own
+    # (matmul_shmem.cu:176-325): all three element types over every legal (tile_dim, block_rows), <int, int> at
+    # tolerance 0, then the TFLOPS lines
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "build", "matmul_shmem_driver")
+    assert os.path.exists(exe), "tests/cpp/build/matmul_shmem_driver is not built (make -C tests/cpp)"
+    r = subprocess.run([exe, "all", "2048"], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "PASSED" in r.stdout and "failed" not in r.stdout
+    for name in ("<half, float>, correctness", "<float, float>, correctness", "<int, int>, correctness", "<int, int>, [TFLOPS]"):
+        assert name in r.stdout
+    passed = [l for l in r.stdout.splitlines() if l.endswith(": passed")]
+    rates = [l for l in r.stdout.splitlines() if l.startswith("(") and "): " in l and not l.endswith("ed")]
+    assert len(passed) >= 3 * 2 * 10 and len(rates) >= 3 * 10 and all(float(l.split("): ")[1]) > 0.1 for l in rates)
