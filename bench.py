@@ -193,6 +193,11 @@ def main():
     ap.add_argument("--no-ceiling", action="store_true", help="skip the bare inner-loop probe of the headline workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
+                    help="ckopt_set_option(KEY, VALUE) before anything is launched (e.g. 0=0: LDS swizzle off, 2=1: no XCD remap, "
+                         "8=0: one barrier per loop body); repeatable")
+    ap.add_argument("--no-vendor", action="store_true",
+                    help="skip timing the vendor library's GEMM (hipBLASLt through torch.mm, fp32 output) on the same operands")
     ap.add_argument("--no-settle", action="store_true",
                     help="skip the set-up launches that bring the device to its sustained clock before warm-up")
     ap.add_argument("--sweep", action="store_true",
@@ -234,6 +239,11 @@ def main():
                           "launches": max(args.steps, 1)}))
         return 0
     cus = args.cus or torch.cuda.get_device_properties(0).multi_processor_count
+    options = {}
+    for kv in args.option:
+        k, v = kv.split("=")
+        ck.set_option(int(k), int(v))
+        options[int(k)] = int(v)
 
     kind, dtype, M, N, K, dist = WORKLOADS[args.workload]
     # tuning flags default to what the library suggests for the shape (ckopt_suggest_gemm_tuning); TUNED records
@@ -412,6 +422,28 @@ def main():
         ceil = mfma_ceiling(1, 1, 400000)
         out["roofline"]["measured_ceiling"] = round(ceil, 1)
         out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
+    if kind == "gemm" and args.workload == "config3_fp16_8192" and not args.no_vendor:
+        # for orientation, outside the timed region: the vendor library's kernel for the same product on the same operands
+        # (fp16 in, fp32 out), timed the same way right after ours, i.e. at the same sustained clock
+        try:
+            ta, tb = da, db.t()
+            for _ in range(3):
+                torch.mm(ta, tb, out_dtype=torch.float32)
+            vev0, vev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            vev0.record(stream)
+            for _ in range(args.steps):
+                vout = torch.mm(ta, tb, out_dtype=torch.float32)
+            vev1.record(stream)
+            torch.cuda.synchronize()
+            vms = vev0.elapsed_time(vev1) / args.steps
+            out["vendor_library"] = {"what": "torch.mm(A, Bt.T, out_dtype=float32) = hipBLASLt, same operands, same steps, timed right "
+                                             "after the timed region", "value": round(flops / (vms * 1e-3) * 1e-12, 2), "unit": "TFLOP/s",
+                                     "ms": round(vms, 5), "max_abs_diff_to_ours": round(float((vout - dd).abs().max()), 6)}
+            del vout
+        except Exception as e:   # an older torch without out_dtype: the comparison is simply left out
+            out["vendor_library"] = {"error": repr(e)[:200]}
+    if options:
+        out["config"]["options"] = options
     if check is not None:
         out["parity_check"] = check
     if not args.no_cpu_baseline:

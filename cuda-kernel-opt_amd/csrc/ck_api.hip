@@ -312,8 +312,9 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     a.bar_steps_b = mode == CK_SYNC_TILE ? 0 : t.bar_steps_b;
     a.swizzle = g_swizzle.load();
     a.num_xcd = g_num_xcd.load();
-    const uintptr_t vec_mask = out16 ? 7 : 15;  // one 8- or 16-byte access per accumulator block
-    a.vec_store = (N % 4 == 0) && !((uintptr_t)D & vec_mask) && (beta == 0.f || !((uintptr_t)C & vec_mask));
+    // one vector access per accumulator block: 16 bytes of fp32 need only the 4-byte alignment checked above
+    // (any N); 8 bytes of 16-bit results need their own alignment
+    a.vec_store = !out16 || ((N % 4 == 0) && !((uintptr_t)D & 7) && (beta == 0.f || !((uintptr_t)C & 7)));
     a.spin_limit = (uint32_t)g_spin_limit.load();
     a.prio_mode = g_prio_mode.load();
     a.producer_nap = g_producer_nap.load();

@@ -207,12 +207,12 @@ __global__ __launch_bounds__(CW * 64) void gemm_fused_kernel(const GemmArgs g) {
         const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
         const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
         const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
-        const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
+        const bool vec_cols = g.vec_store && (rc.col + 1) * TILE <= g.N;
 #pragma unroll
         for (int i = 0; i < WTR; ++i) {
 #pragma unroll
             for (int j = 0; j < WTC; ++j) {
-                epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
+                epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], vec_cols);
                 acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }

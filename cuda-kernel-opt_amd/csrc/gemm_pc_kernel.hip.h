@@ -39,6 +39,9 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// Four fp32 results of one output row as ONE 16-byte access at an address that is only 4-byte aligned (rows of D
+// start anywhere when N is not a multiple of 4): global dwordx4 accesses need dword alignment, not 16 bytes.
+typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));
 
 #define CK_LDS __attribute__((address_space(3)))
 
@@ -58,7 +61,7 @@ struct GemmArgs {
     int bar_steps_a, bar_steps_b;
     int swizzle;
     int num_xcd;
-    int vec_store;  // D (and C) aligned for one vector access per accumulator block, N % 4 == 0
+    int vec_store;  // C and D allow one vector access per accumulator block (fp32: always; 16-bit: N % 4 == 0, 8-byte aligned)
     int out16;      // C and D hold the operands' 16-bit element type instead of fp32 (accumulation stays fp32)
     int split_k;    // straight-line kernel only: K is cut into this many slices (>= 1), one work item per (tile, slice);
                     // slice s writes its partial products to D + s * M * N (a workspace; alpha 1, beta 0, fp32)
@@ -103,17 +106,20 @@ template <> struct Out16<bf16_tag> {
         return (unsigned short)(u >> 16);
     }
 };
+// vec_cols: the tile's columns all lie inside the matrix and C / D allow one vector access per block (fp32: always;
+// 16-bit: N % 4 == 0 and 8-byte aligned pointers); rows past M are skipped. Otherwise element by element.
 template <typename DT>
-__device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, f32x4 acc, bool interior) {
+__device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, f32x4 acc, bool vec_cols) {
     const int64_t off = (int64_t)m * g.N + n;
     const float alpha = g.alpha, beta = g.beta;
     f32x4 v = acc * alpha;
+    if (m >= g.M) return;
     if (!g.out16) {
-        if (interior) {
-            if (beta != 0.f) v += *(const f32x4*)(g.C + off) * beta;
+        if (vec_cols) {
+            if (beta != 0.f) v += *(const f32x4_u*)(g.C + off) * beta;
             // D is written once and not read again: non-temporal, so that it does not displace the operands in L2
-            __builtin_nontemporal_store(v, (f32x4*)(g.D + off));
-        } else if (m < g.M) {
+            __builtin_nontemporal_store(v, (f32x4_u*)(g.D + off));
+        } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 if (n + e < g.N) {
@@ -126,7 +132,7 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
     } else {
         const unsigned short* c16 = (const unsigned short*)g.C;
         unsigned short* d16 = (unsigned short*)g.D;
-        if (interior) {
+        if (vec_cols) {
             if (beta != 0.f) {
                 const uint2 c = *(const uint2*)(c16 + off);
                 v[0] += Out16<DT>::load((unsigned short)(c.x & 0xffffu)) * beta;
@@ -139,7 +145,7 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
             o.y = (uint32_t)Out16<DT>::store(v[2]) | ((uint32_t)Out16<DT>::store(v[3]) << 16);
             typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
             __builtin_nontemporal_store(u32x2{o.x, o.y}, (u32x2*)(d16 + off));
-        } else if (m < g.M) {
+        } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 if (n + e < g.N) {
@@ -610,11 +616,11 @@ __device__ __forceinline__ void consume(const GemmArgs& g, uint32_t flags_base, 
         // fragment as the first MFMA operand a lane holds 4 consecutive columns of one row.
         const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
         const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
-        const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
+        const bool vec_cols = g.vec_store && (rc.col + 1) * TILE <= g.N;
 #pragma unroll
         for (int i = 0; i < WTR; ++i) {
 #pragma unroll
-            for (int j = 0; j < WTC; ++j) epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
+            for (int j = 0; j < WTC; ++j) epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], vec_cols);
         }
     }
 }

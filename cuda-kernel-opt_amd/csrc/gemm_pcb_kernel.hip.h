@@ -168,11 +168,11 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_pcb_kernel(const GemmArgs g) {
             }
             const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
             const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
-            const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
+            const bool vec_cols = g.vec_store && (rc.col + 1) * TILE <= g.N;
 #pragma unroll
             for (int i = 0; i < WTR; ++i) {
 #pragma unroll
-                for (int j = 0; j < WTC; ++j) epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
+                for (int j = 0; j < WTC; ++j) epilogue_block<DT>(g, m_base + i * 16, n_base + j * 16, acc[i][j], vec_cols);
             }
         }
         if (blockIdx.x == 0 && threadIdx.x == blockDim.x - 1) {

@@ -291,8 +291,12 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             go.D = g.D + (size_t)slice * ((size_t)g.M * g.N);
             const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
             const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
-            const bool interior = g.vec_store && (rc.row + 1) * TILE <= g.M && (rc.col + 1) * TILE <= g.N;
-            if (interior && !g.out16) {
+            // vec_cols: every column of the tile is inside the matrix, one vector access per block (rows past M are
+            // skipped lane by lane); interior: every row as well, so every wave issues exactly the stores that the next
+            // body's landing wait counts
+            const bool vec_cols = g.vec_store && (rc.col + 1) * TILE <= g.N;
+            const bool interior = vec_cols && (rc.row + 1) * TILE <= g.M;
+            if (vec_cols && !g.out16) {
                 // Whole 128-byte lines per store: an accumulator block gives a row 64 bytes (4 lanes x 16),
                 // and the write path's cost is per request, not per byte. Two neighbouring blocks are
                 // exchanged between lanes so that 8 lanes hold the 32 consecutive floats of one row:
@@ -318,9 +322,12 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                                 const int a1 = __builtin_amdgcn_ds_bpermute(src0 + tt * 32, __float_as_int(x1));
                                 v[e] = __int_as_float(second ? a1 : a0) * alpha;
                             }
-                            const int64_t off = (row0 + i * 16 + tt * 8) * g.N + (col0 + j * 16);
-                            if (beta != 0.f) v += *(const f32x4*)(go.C + off) * beta;
-                            __builtin_nontemporal_store(v, (f32x4*)(go.D + off));
+                            const int64_t row = row0 + i * 16 + tt * 8;
+                            const int64_t off = row * g.N + (col0 + j * 16);
+                            if (row < g.M) {
+                                if (beta != 0.f) v += *(const f32x4_u*)(go.C + off) * beta;
+                                __builtin_nontemporal_store(v, (f32x4_u*)(go.D + off));
+                            }
                         }
                     }
                 }
@@ -374,7 +381,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
                 for (int i = 0; i < WTR; ++i)
 #pragma unroll
-                    for (int j = 0; j < WTC; ++j) epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], interior);
+                    for (int j = 0; j < WTC; ++j) epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], vec_cols);
             }
 #pragma unroll
             for (int i = 0; i < WTR; ++i)

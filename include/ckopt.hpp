@@ -11,6 +11,7 @@
 #ifndef CKOPT_HPP
 #define CKOPT_HPP
 
+#include <cstddef>
 #include <cstdint>
 #include <stdexcept>
 #include <string>
@@ -28,6 +29,21 @@ struct Error : std::runtime_error {
     Error(int c, const char* where) : std::runtime_error(std::string(where) + ": " + ckopt_error_string(c)), code(c) {}
 };
 inline void check(int rc, const char* where) { if (rc != CKOPT_OK) throw Error(rc, where); }
+
+// The kernels' flag waits are bounded: a wave that gives one up sets a status bit and the launch's D is then invalid
+// (cuda::barrier waits in the reference are unbounded and would hang instead). The launcher templates below do not
+// synchronise, so they cannot report it; a caller that wants the check calls this after its launches: it waits for
+// `stream`, reads and clears the device's status word and throws if a wait was given up.
+struct DeviceStatusError : std::runtime_error {
+    int status;
+    explicit DeviceStatusError(int s)
+        : std::runtime_error("a bounded flag wait was given up (device status " + std::to_string(s) + "): results are invalid"), status(s) {}
+};
+inline void synchronize_and_check(void* stream = nullptr) {
+    const int st = ckopt_device_status(stream);
+    if (st < 0) throw Error(st, "device_status");
+    if (st != 0) throw DeviceStatusError(st);
+}
 
 inline float to_float(float x) { return x; }
 inline float to_float(half_t x) { return (float)x; }
@@ -64,6 +80,19 @@ void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B /* transposed: N x K 
                                                       num_consumer_warps, num_sms, stream),
               "gemm_shmem_tc_async_opt_port <DT, DT>");
     }
+}
+// port_2 on caller-owned scratch memory (ckopt_gemm_workspace_bytes says how much): nothing is allocated
+template <typename DT, typename DT_ACC>
+void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B, const DT_ACC* C, DT_ACC* D, DT_ACC alpha, DT_ACC beta, int M, int N, int K,
+                                  int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                                  int bar_step_rows_b, int tile_group_m, int num_stages, int num_producer_warps, int num_consumer_warps,
+                                  int num_sms, void* workspace, std::size_t workspace_bytes, void* stream) {
+    static_assert(std::is_same<DT_ACC, float>::value || std::is_same<DT_ACC, DT>::value, "C / D are fp32 or the operand type");
+    check(ckopt_gemm_shmem_tc_async_opt_port_2_ws(dtype_of<DT>::value, dtype_of<DT_ACC>::value, A, B, C, D, to_float(alpha), to_float(beta), M, N,
+                                                  K, tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                                                  tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, workspace,
+                                                  workspace_bytes, stream),
+          "gemm_shmem_tc_async_opt_port (workspace)");
 }
 // port_1: granularity only
 template <typename DT, typename DT_ACC>
