@@ -303,25 +303,31 @@ def main():
 
     # Set-up, outside warm-up and the timed region: bring the device to the state a running job sees. A fresh
     # process finds the device idle at its top clock; under the matrix cores' load the power controller first
-    # undershoots (launches 3 to 6 take 1.1 ms at 8192^3) and needs about 50 launches to come back to the clock it
-    # then holds (0.79 ms). Batches of launches are repeated until two consecutive batches agree within 1 %.
+    # undershoots (launches 3 to 6 take 1.1 ms at 8192^3) and needs about 50 ms to come back to the clock it
+    # then holds (0.79 ms). Batches of about 25 ms of launches are repeated until two consecutive batches agree
+    # within 1 % (at least 75 ms in all).
     settle = {"launches": 0, "first_batch_ms": None, "last_batch_ms": None}
     if not args.no_settle:
-        batch = max(4, min(20, int(20e-3 / max(2.0 * M * N * K / 1.2e15, 1e-5))))   # about 20 ms of launches
-        prev = None
         sev0, sev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for _ in range(30):
+
+        def timed_batch(n):
             sev0.record(stream)
-            for _ in range(batch):
+            for _ in range(n):
                 step()
             sev1.record(stream)
             sev1.synchronize()
-            cur = sev0.elapsed_time(sev1) / batch
-            settle["launches"] += batch
-            if settle["first_batch_ms"] is None:
-                settle["first_batch_ms"] = round(cur, 5)
+            settle["launches"] += n
+            return sev0.elapsed_time(sev1) / n
+
+        settle["first_batch_ms"] = round(timed_batch(4), 5)    # cold: includes the runtime's first-launch work
+        cur = timed_batch(4)
+        batch = max(4, min(400, int(25.0 / max(cur, 1e-3))))   # about 25 ms of launches: the controller's time scale
+        prev, spent_ms = None, 0.0
+        for _ in range(40):
+            cur = timed_batch(batch)
+            spent_ms += cur * batch
             settle["last_batch_ms"] = round(cur, 5)
-            if prev is not None and settle["launches"] >= 3 * batch and abs(cur - prev) <= 0.01 * prev:
+            if prev is not None and spent_ms >= 75.0 and abs(cur - prev) <= 0.01 * prev:
                 break
             prev = cur
 
@@ -427,7 +433,7 @@ def main():
         # (fp16 in, fp32 out), timed the same way right after ours, i.e. at the same sustained clock
         try:
             ta, tb = da, db.t()
-            for _ in range(3):
+            for _ in range(100):   # the other kernel draws different power: let the clock find its level again
                 torch.mm(ta, tb, out_dtype=torch.float32)
             vev0, vev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             vev0.record(stream)

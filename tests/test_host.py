@@ -263,3 +263,31 @@ def test_matmul_shmem_multiply_adds_avoid_one_bank_operands(tmp_path):
         assert not bad, "%s: %d of %d multiply-adds with all registers in one bank" % (name, len(bad), len(ops))
         checked += 1
     assert checked >= 16
+
+
+def test_workspace_query_follows_the_launcher_rules(ck):
+    # pure host arithmetic (no GPU call): what a launch takes from a caller-owned workspace
+    straight = (256, 32, 0, 0, 256, 256, 4, 5, 0, 8, 256)
+    pc = (128, 64, 0, 0, 128, 128, 4, 2, 2, 4, 256)
+    r256 = lambda n: (n + 255) // 256 * 256
+    # aligned operands, enough tiles: nothing
+    assert ck.gemm_workspace_bytes(8192, 8192, 8192, True, *straight) == 0
+    assert ck.gemm_workspace_bytes(512, 512, 512, True, *pc) == 0
+    # config 4: 64 tiles on 256 CUs -> four slices of 2048 x 2048 fp32, plus room to align the caller's pointer
+    assert ck.gemm_workspace_bytes(2048, 2048, 32768, True, *straight) == 4 * 2048 * 2048 * 4 + 256
+    # config 5: rows of 3071 elements -> zero-padded copies of both operands with rows of 3072; 408 tiles are not cut
+    assert ck.gemm_workspace_bytes(6143, 4097, 3071, True, *straight) == r256((6143 + 4097) * 3072 * 2) + 256
+    # operands off a 16-byte boundary are copied whatever K is; other kernels never cut K
+    assert ck.gemm_workspace_bytes(512, 512, 512, False, *pc) == r256(2 * 512 * 512 * 2) + 256
+    assert ck.gemm_workspace_bytes(256, 256, 32768, True, *pc) == 0
+    # copies and planes together (2 x 3 tiles, K 4090 -> 4096, four slices)
+    assert ck.gemm_workspace_bytes(300, 520, 4090, True, *straight) == r256((300 + 520) * 4096 * 2) + r256(4 * 300 * 520 * 4) + 256
+    # the split-K switch is part of the rule
+    prev = ck.set_option(ck.OPT_SPLIT_K, 0)
+    try:
+        assert ck.gemm_workspace_bytes(2048, 2048, 32768, True, *straight) == 0
+    finally:
+        ck.set_option(ck.OPT_SPLIT_K, prev)
+    for bad in ((0, 1, 1), (1, 0, 1), (1, 1, 0)):
+        with pytest.raises(ck.CkoptError):
+            ck.gemm_workspace_bytes(*bad, True, *straight)
