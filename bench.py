@@ -287,7 +287,7 @@ def main():
                                             args.producers, args.consumers, cus, stream)
         peak, bound_name, arith = PEAK_TFLOPS["mfma_f16"], "mfma", dtype
         if (args.producers == 0 and args.tile == 256 and args.segk == 32 and args.stages == 5 and args.consumers == 8
-                and (K + 7) // 8 * 8 % 64 == 0):
+                and options.get(6, 1) and options.get(0, 1)):
             kernel = "gemm_stream_kernel<%s, tile 256, five 32-deep quarters, 8 waves, pair fetch>" % dtype
         elif args.producers == 0:
             kernel = "gemm_fused_kernel<%s, tile %d, seg_k %d, %d waves, workgroup barrier per segment>" % (

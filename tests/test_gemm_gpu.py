@@ -553,6 +553,25 @@ def test_straight_line_kernel_bit_exact(ck, M, N, K, cus, group):
             assert np.array_equal(got, want), every_kstep
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 260, 200), (512, 256, 8), (256, 520, 1001), (130, 70, 4100)])
+def test_straight_line_kernel_any_k(ck, M, N, K):
+    # K that is not a multiple of 64 (or of 8): the operand copies pad the rows with zeros to whole loop bodies, and the
+    # launch still takes the straight-line kernel; exact on small integers, with and without C, every element written
+    for dt in (ck.DT_F16, ck.DT_BF16):
+        a = ck.fill_int(dt, (M, K), 98, 0, -2, 2)
+        bt = ck.fill_int(dt, (N, K), 98, 1, -2, 2)
+        c = ck.fill_int(ck.DT_F32, (M, N), 98, 2, -3, 3)
+        exact = G.as_f64(dt == ck.DT_BF16, a) @ G.as_f64(dt == ck.DT_BF16, bt).T
+        for cus in (256, 3):
+            t = _straight_line_tuning(ck, cus)
+            assert np.array_equal(G.run_gemm(ck, dt, a, bt, t=t), exact.astype(np.float32)), (M, N, K, dt, cus)
+            assert np.array_equal(G.run_gemm(ck, dt, a, bt, c, -1.0, 2.0, t=t), (2.0 * c - exact).astype(np.float32))
+    order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b",
+                            "tile_group_m", "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
+    if K % 64:
+        assert ck.gemm_workspace_bytes(M, N, K, True, *order) >= (M + N) * ((K + 63) // 64 * 64) * 2
+
+
 @pytest.mark.parametrize("M,N,K,cus", [
     (1280, 1280, 192, 24),   # 25 tiles on 24 workgroups: 2 rounds, even rounds take 16 workgroups
     (1279, 1025, 320, 12),   # ragged, 25 tiles on 12: 3 rounds, 9 -> 12 workgroups (rounded up to whole XCDs, capped)

@@ -228,7 +228,12 @@ def test_suggested_tunings_are_legal_and_follow_the_measured_rules(ck):
     assert picks(1024, 1024, 8192) == straight          # 16 tiles, eight slices of 1024
     assert picks(2048, 2048, 2048)["tile_dim"] == 128   # 64 tiles of 256 and K too shallow to cut four times
     assert picks(512, 512, 512)["tile_dim"] == 64       # config 1
-    assert picks(8192, 8192, 8200)["num_producer_warps"] == 2 and picks(8192, 8192, 8200)["tile_dim"] == 256  # K % 64 != 0
+    assert picks(8192, 8192, 8200) == straight          # any K: the operand copies pad it to whole loop bodies of 64
+    prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
+    try:
+        assert picks(8192, 8192, 8192)["num_producer_warps"] == 2 and picks(8192, 8192, 8192)["tile_dim"] == 256
+    finally:
+        ck.set_option(ck.OPT_STRAIGHT_LINE, prev)
     with pytest.raises(ck.CkoptError):
         ck.suggest_gemm_tuning(0, 1, 1)
 
@@ -282,6 +287,9 @@ def test_workspace_query_follows_the_launcher_rules(ck):
     assert ck.gemm_workspace_bytes(256, 256, 32768, True, *pc) == 0
     # copies and planes together (2 x 3 tiles, K 4090 -> 4096, four slices)
     assert ck.gemm_workspace_bytes(300, 520, 4090, True, *straight) == r256((300 + 520) * 4096 * 2) + r256(4 * 300 * 520 * 4) + 256
+    # K 8200 with the straight-line tuple: copies with rows of 8256 (whole loop bodies of 64); other tuples need none
+    assert ck.gemm_workspace_bytes(8192, 8192, 8200, True, *straight) == r256(2 * 8192 * 8256 * 2) + 256
+    assert ck.gemm_workspace_bytes(8192, 8192, 8200, True, *pc) == 0
     # the split-K switch is part of the rule
     prev = ck.set_option(ck.OPT_SPLIT_K, 0)
     try:
