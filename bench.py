@@ -72,6 +72,20 @@ def mfma_ceiling(random_operands, with_loads, ksteps=400000):
     return out.value
 
 
+def valu_ceiling(random_operands, iters=400000):
+    """TFLOP/s of the bare fp32 multiply-add stream of the matmul_shmem micro-tile on every CU (no LDS, no loads):
+    int ckmeasure_valu_ceiling(int random_operands, int iters, double* tflops_out) of libckmeasure.so."""
+    import ctypes
+    lib = ctypes.CDLL(os.path.join(ROOT, "cuda-kernel-opt_amd", "lib", "libckmeasure.so"))
+    lib.ckmeasure_valu_ceiling.restype = ctypes.c_int
+    lib.ckmeasure_valu_ceiling.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    out = ctypes.c_double(0.0)
+    rc = lib.ckmeasure_valu_ceiling(int(bool(random_operands)), int(iters), ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError("ckmeasure_valu_ceiling failed (%d)" % rc)
+    return out.value
+
+
 def cpu_baseline(ck, kind, dtype, a, b, M, N, K, budget_s=12.0):
     """Times the CPU oracle on a bounded row sample of the same operands; returns the JSON object."""
     from oracle import oracle as o
@@ -225,6 +239,7 @@ def main():
             for loads in (0, 1):
                 key = "%s_operands_%s" % ("random" if rnd else "constant", "with_loads" if loads else "no_loads")
                 res[key] = round(mfma_ceiling(rnd, loads, 400000), 1)
+            res["fp32_valu_%s_operands" % ("random" if rnd else "constant")] = round(valu_ceiling(rnd), 1)
         print(json.dumps({"probe": "bare inner loop of the 256x256 tile GEMM, 8 waves per CU, ~0.2 s per case",
                           "unit": "TFLOP/s", "nominal_peak": PEAK_TFLOPS["mfma_f16"], **res}))
         return 0
@@ -412,7 +427,8 @@ def main():
         "pct_of_peak": round(100.0 * value / peak, 2),
         "config": {"workload": "%s: %s %dx%dx%d, A MxK and Bt NxK row-major, %s inputs from seed, fp32 accumulate/output"
                                % (args.workload, dtype, M, N, K, "uniform[-1,1)" if dist == "uniform" else "N(0,1)*0.1"),
-                   "kernel": kernel, "tile_group_m": args.group, "num_stages": args.stages, "grid_cus": cus},
+                   "kernel": kernel, **({"tile_group_m": args.group, "num_stages": args.stages, "grid_cus": cus} if kind == "gemm" else
+                                        {"tile_dim": args.simt_tile, "block_rows": args.block_rows, "b_transposed": True})},
         "roofline": {"bound": "mfma" if bound_name == "mfma" else "valu", "achieved": round(achieved, 2), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(achieved / peak, 4), "traffic": traffic,
                      "traffic_source": None if traffic is None else "recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
@@ -426,6 +442,11 @@ def main():
         # loads of the real data flow (no synchronisation, no waiting, no epilogue): the device's power limit
         # keeps it well below the nominal peak, and no kernel of this shape can exceed it
         ceil = mfma_ceiling(1, 1, 400000)
+        out["roofline"]["measured_ceiling"] = round(ceil, 1)
+        out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
+    if kind == "simt" and not args.no_ceiling:
+        # the same for the vector ALUs: the micro-tile's multiply-add stream with random operands and nothing to feed it
+        ceil = valu_ceiling(1)
         out["roofline"]["measured_ceiling"] = round(ceil, 1)
         out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
     if kind == "gemm" and args.workload == "config3_fp16_8192" and not args.no_vendor:

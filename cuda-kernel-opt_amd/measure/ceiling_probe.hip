@@ -114,7 +114,84 @@ hipError_t launch_probe(int cus, const char* window, int ksteps, float* sink, hi
     return hipGetLastError();
 }
 
+// The fp32 vector ALUs alone: what the matmul_shmem kernel's multiply-add stream sustains when nothing feeds it (no
+// LDS reads, no global loads, no barrier). 512 threads per workgroup, four workgroups per CU (eight waves per SIMD, the
+// kernel's occupancy); per thread an 8 x 4 accumulator micro-tile in registers and 32 v_fmac_f32 per iteration on 8 + 4
+// operand registers. Accumulator rows and the B values are even-aligned runs of four registers with column j of an
+// accumulator row in element j + 1, as in the kernel, so that no multiply-add has its three registers in one bank
+// (those run at half rate).
+typedef float probe_f4 __attribute__((ext_vector_type(4)));
+template <bool RANDOM>
+__global__ __launch_bounds__(512) void valu_probe_kernel(int iters, float* sink) {
+    const uint32_t tid = blockIdx.x * 512u + threadIdx.x;
+    float a[8];
+    probe_f4 b, acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        uint32_t h = (tid * 8u + i) * 2654435761u;
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+        a[i] = RANDOM ? (float)(h >> 8) * (2.0f / 16777216.0f) - 1.0f : 1.0f;
+        acc[i] = probe_f4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t h = (tid * 4u + j + 977u) * 2246822519u;
+        h ^= h >> 15; h *= 2654435761u; h ^= h >> 13;
+        b[j] = RANDOM ? (float)(h >> 8) * (2.0f / 16777216.0f) - 1.0f : 1.0f;
+    }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) asm volatile("" : "+v"(acc[i]));
+        asm volatile("" : "+v"(b));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            asm volatile("" : "+v"(a[i]));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][(j + 1) % 4] = __builtin_fmaf(a[i], b[j], acc[i][(j + 1) % 4]);
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    sink[tid] = s;
+}
+
 }  // namespace
+
+// TFLOP/s of the bare fp32 multiply-add stream on every CU (see valu_probe_kernel): iters iterations of 32
+// multiply-adds per thread after a warm-up; random_operands selects random instead of constant operand values.
+extern "C" int ckmeasure_valu_ceiling(int random_operands, int iters, double* tflops_out) {
+    using namespace ck;
+    if (!tflops_out || iters < 2 || iters > (1 << 28)) return CK_ERR_BAD_PARAM;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return CK_ERR_HIP;
+    const int blocks = cus * 4;
+    float* sink = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int rc = CK_ERR_HIP;
+    do {
+        if (hipMalloc((void**)&sink, (size_t)blocks * 512 * sizeof(float)) != hipSuccess) break;
+        if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) break;
+        auto go = [&](int n) {
+            if (random_operands) hipLaunchKernelGGL(valu_probe_kernel<true>, dim3(blocks), dim3(512), 0, nullptr, n, sink);
+            else hipLaunchKernelGGL(valu_probe_kernel<false>, dim3(blocks), dim3(512), 0, nullptr, n, sink);
+            return hipGetLastError();
+        };
+        if (go(iters / 4 + 2) != hipSuccess) break;   // warm-up
+        if (hipEventRecord(e0, nullptr) != hipSuccess) break;
+        if (go(iters) != hipSuccess) break;
+        if (hipEventRecord(e1, nullptr) != hipSuccess || hipEventSynchronize(e1) != hipSuccess) break;
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess || ms <= 0.f) break;
+        *tflops_out = (double)blocks * 512.0 * iters * 32.0 * 2.0 / (ms * 1e-3) * 1e-12;
+        rc = CK_OK;
+    } while (false);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (sink) (void)hipFree(sink);
+    return rc;
+}
 
 // Built into lib/libckmeasure.so, a measurement aid that bench.py loads next to the product library (which does not
 // contain it). random_operands: random instead of constant fragment values; with_loads: also the direct-to-LDS loads;
