@@ -175,7 +175,10 @@ int ckopt_device_status(void* stream);
  * matrix-core utilisation. No reference counterpart. */
 int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* ref_ticks);
 
-/* Process-wide tuning switches that are not launcher parameters in the reference:
+/* Process-wide tuning switches that are not launcher parameters in the reference. Each is one atomic word that a
+ * launch reads once; a switch changed by one thread while another launches takes effect for either all or none of
+ * that launch, but two threads that need different settings at the same time must serialise their set / launch pairs
+ * themselves (the reference's launchers have no such state: every knob there is a parameter).
  * key 0: LDS XOR swizzle on/off (default 1); key 1: spin limit of bounded waits (default 1<<22);
  * key 2: number of XCDs assumed by the workgroup->tile remap (default 8; 1 disables the remap);
  * key 3: wave priorities of the counter-synchronised kernel (0 producers raised (default), 1 also asymmetric

@@ -299,3 +299,12 @@ def test_workspace_query_follows_the_launcher_rules(ck):
     for bad in ((0, 1, 1), (1, 0, 1), (1, 1, 0)):
         with pytest.raises(ck.CkoptError):
             ck.gemm_workspace_bytes(*bad, True, *straight)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # every box of this build has one GPU and the GEMM path has no collective: --gpus 2 exits with a message that says so
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
