@@ -238,10 +238,8 @@ bool straight_line_tuple(const ck::GemmTuning& t) {
     return g_straight_line.load() && g_swizzle.load() && t.num_producer_waves == 0 && t.num_consumer_waves == 8 && t.tile_dim == 256 &&
            t.segment_dim_k == 32 && t.num_stages == 5;
 }
-// K as the kernels see it: operand rows are zero-padded to whole 16-byte chunks, and for the straight-line tuple to
-// whole loop bodies, so that any K takes that kernel: the copy reads and writes (M + N) * K * 2 bytes and still pays
-// (fp16 8192^2 x 8200: 1218 TFLOP/s with the copies against 1153 for the general fused kernel on the operands as
-// they are; x 3000: 1133 against 1044).
+// K of the zero-padded operand copies (made when K % 8 != 0 or an operand is off a 16-byte boundary): whole 16-byte
+// chunks, and for the straight-line tuple whole loop bodies, so that the copies take that kernel's plain instance.
 int padded_k(int K, const ck::GemmTuning& t) {
     const int unit = straight_line_tuple(t) ? ck::STREAM_K_MULTIPLE_HOST : ck::CHUNK_ELEMS;
     return (K + unit - 1) / unit * unit;
@@ -254,7 +252,7 @@ size_t scratch_need(int M, int N, int K, bool operands_aligned, const ck::GemmTu
     using namespace ck;
     size_t need = 0;
     int k = K;
-    if (K != padded_k(K, t) || !operands_aligned) {
+    if (K % CHUNK_ELEMS != 0 || !operands_aligned) {
         k = padded_k(K, t);
         need += scratch_round(((size_t)M + (size_t)N) * k * 2);
     }
@@ -302,7 +300,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     const uintptr_t elem_mask = out16 ? 1 : 3;
     if (((uintptr_t)D & elem_mask) || ((uintptr_t)C & elem_mask)) return CK_ERR_ALIGNMENT;
     // the kernels want every operand row on a 16-byte boundary
-    if (K != padded_k(K, t) || ((uintptr_t)A & 15) || ((uintptr_t)Bt & 15))
+    if (K % CHUNK_ELEMS != 0 || ((uintptr_t)A & 15) || ((uintptr_t)Bt & 15))
         return gemm_launch_repacked(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, out16, sc);
     // one tile's rows are addressed through a 32-bit buffer offset
     if ((int64_t)t.tile_dim * K * 2 >= (int64_t)1 << 31) return CK_ERR_TOO_LARGE;

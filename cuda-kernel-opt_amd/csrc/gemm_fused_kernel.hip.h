@@ -45,6 +45,17 @@ __device__ __forceinline__ void dma_load_b128(i32x4 rsrc, uint32_t lds_dst, uint
                  : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff)
                  : "memory");
 }
+// The same load with one of two per-lane offsets, chosen by a wave-uniform flag through a scalar branch inside the
+// statement (a select in vector registers would put a vector ALU instruction in front of every load, and those share
+// the matrix cores' issue port; a branch the compiler can see would split the caller's loop body into basic blocks).
+__device__ __forceinline__ void dma_load_b128_select(i32x4 rsrc, uint32_t lds_dst, uint32_t voff, uint32_t voff_if_flag, uint32_t soff,
+                                                     uint32_t flag) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_cmp_lg_u32 %5, 0\n\ts_cbranch_scc1 1f\n\tbuffer_load_dwordx4 %1, %3, %4 offen lds\n\ts_branch 2f\n1:\n\t"
+                 "buffer_load_dwordx4 %2, %3, %4 offen lds\n2:"
+                 :
+                 : "s"(lds_dst), "v"(voff), "v"(voff_if_flag), "s"(rsrc), "s"(soff), "s"(flag)
+                 : "memory", "scc");
+}
 __device__ __forceinline__ i32x4 make_rsrc(const void* base, uint32_t num_records) {
     const uint64_t p = (uint64_t)(uintptr_t)base;
     i32x4 r;

@@ -5,9 +5,9 @@ namespace ck {
 
 static_assert(STREAM_K_MULTIPLE == 64, "the host's slice rule assumes loop bodies of 64");
 
-template <typename DT, bool ODD_ONLY>
-static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a) {
-    auto kern = gemm_stream_kernel<DT, ODD_ONLY>;
+template <typename DT, bool ODD_ONLY, bool KTAIL>
+static hipError_t stream_launch_one(dim3 grid, hipStream_t stream, const GemmArgs& a) {
+    auto kern = gemm_stream_kernel<DT, ODD_ONLY, KTAIL>;
     static bool opted[64] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -21,6 +21,12 @@ static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a
     return hipGetLastError();
 }
 
+// K in whole loop bodies: the plain instance; otherwise (K a multiple of 8) the one whose last body masks the end of K
+template <typename DT, bool ODD_ONLY>
+static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a) {
+    return a.K % STREAM_K_MULTIPLE == 0 ? stream_launch_one<DT, ODD_ONLY, false>(grid, stream, a) : stream_launch_one<DT, ODD_ONLY, true>(grid, stream, a);
+}
+
 // barrier_every_kstep selects the schedule with a barrier in both k-steps of a loop body
 hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep) {
     return barrier_every_kstep ? stream_launch<f16_tag, false>(grid, stream, a) : stream_launch<f16_tag, true>(grid, stream, a);
@@ -32,7 +38,7 @@ hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs
 // what the kernel assumes about a launch (the caller falls back to the general fused kernel otherwise)
 bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves) {
     return producer_waves == 0 && consumer_waves == 8 && tile_dim == STREAM_TILE && segment_dim_k == STREAM_SEGK &&
-           num_stages == STREAM_STAGES && a.K % STREAM_K_MULTIPLE == 0 && a.swizzle;
+           num_stages == STREAM_STAGES && a.K % CHUNK_ELEMS == 0 && a.swizzle;
 }
 
 }  // namespace ck

@@ -49,7 +49,11 @@ constexpr int STREAM_STAGES = 5;
 constexpr int STREAM_K_MULTIPLE = 2 * STREAM_SEGK;  // one loop body
 constexpr int STREAM_LDS_BYTES = STREAM_STAGES * 2 * STREAM_TILE * STREAM_SEGK * 2;
 
-template <typename DT, bool ODD_ONLY>
+// KTAIL: K is a multiple of 8 but not of 64. The last loop body of a tile then reaches past K: its loads take
+// per-lane offsets in which every 16-byte chunk at or beyond K lies outside the descriptor (reads as zeros), chosen
+// by a scalar branch inside the load's asm statement, so that nothing is added to the other bodies but two scalar
+// instructions per load. Launches with K % 64 == 0 run the instance without any of it.
+template <typename DT, bool ODD_ONLY, bool KTAIL>
 __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     constexpr int TILE = STREAM_TILE, NQ = STREAM_STAGES;
     constexpr int WTR = 4, WTC = 8;          // 16 x 16 blocks per wave tile (64 x 128)
@@ -88,9 +92,9 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     const int S = g.split_k;
     const int total_items = g.tiles_m * g.tiles_n * S;
     const int my_tiles = slot < total_items ? (total_items - slot + grid - 1) / grid : 0;
-    const int kslice = g.K / S;                  // the host makes this a multiple of one loop body
+    const int kslice = g.K / S;                  // the host makes this a multiple of one loop body (KTAIL: S is 1, of 8)
     const uint32_t kslice_bytes = (uint32_t)kslice * 2u;
-    const int nb = kslice / STREAM_K_MULTIPLE;   // loop bodies per item
+    const int nb = (kslice + STREAM_K_MULTIPLE - 1) / STREAM_K_MULTIPLE;   // loop bodies per item
     const int CH = g.split_chunk;
     auto item_tile = [&](int64_t item, int& slice) __attribute__((always_inline)) {
         const int64_t chunk = item / CH;
@@ -110,6 +114,21 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     // unchecked scalar offset.
     const uint32_t loff_lo = (uint32_t)(wave * 16 + lane_row) * pitch32 + (uint32_t)swizzle_slot(lane_row, lane_slot, 4, 1) * CHUNK_BYTES;
     const uint32_t loff_hi = loff_lo + 8u * 16u * pitch32;   // rows 16(w+8)..
+    // KTAIL: the same offsets for the body that holds the end of K (rem of its 64 k exist): a lane whose chunk starts at
+    // or beyond rem gets an offset outside any descriptor, per half (first / second 32 k) of the body
+    uint32_t toff_lo[2] = {0, 0}, toff_hi[2] = {0, 0};
+    if constexpr (KTAIL) {
+        const int rem = kslice % STREAM_K_MULTIPLE;
+        const int chunk_k = swizzle_slot(lane_row, lane_slot, 4, 1) * CHUNK_ELEMS;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const bool absent = h * STREAM_SEGK + chunk_k >= rem;
+            toff_lo[h] = absent ? 0x7fffff00u : loff_lo;
+            toff_hi[h] = absent ? 0x7fffff00u : loff_hi;
+        }
+    }
+    uint32_t l_tail = 0;  // KTAIL: nonzero while the body being loaded is the one that holds the end of K
+    if constexpr (KTAIL) asm volatile("s_mov_b32 %0, %1" : "=s"(l_tail) : "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kslice <= STREAM_K_MULTIPLE))));
     const uint32_t dst_w = ring_base + (uint32_t)wave * 1024u;
     i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // empty descriptors: loads read zeros
     uint32_t l_koff = 0;  // byte offset along K of the body being loaded
@@ -132,11 +151,13 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     };
     auto loader_advance = [&]() __attribute__((always_inline)) {
         l_koff += STREAM_K_MULTIPLE * 2;
-        if (l_koff == kslice_bytes) {
+        if (l_koff >= kslice_bytes) {
             l_koff = 0;
             ++l_tile;
             loader_open_tile();
         }
+        if constexpr (KTAIL)   // (kept in one opaque scalar register, like stores_in_flight below)
+            asm volatile("s_mov_b32 %0, %1" : "=s"(l_tail) : "s"(__builtin_amdgcn_readfirstlane((uint32_t)(l_koff + STREAM_K_MULTIPLE * 2 > kslice_bytes))));
     };
     // Load pair P (0, 1: A rows 16w.. / 16(w+8)..; 2, 3: Bt likewise) of the body at l_koff: the two
     // halves of each row's line, back to back, into the quarters at byte offsets q_lo and q_hi.
@@ -145,8 +166,14 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         constexpr bool IS_A = P < 2;
         constexpr int HI = P % 2;
         const uint32_t dst = dst_w + (uint32_t)((IS_A ? 0 : OPB) + HI * 8 * 1024);
-        dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_lo, HI ? loff_hi : loff_lo, l_koff);
-        dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_hi, HI ? loff_hi : loff_lo, l_koff + (uint32_t)(STREAM_SEGK * 2));
+        if constexpr (KTAIL) {
+            dma_load_b128_select(IS_A ? rsrc_a : rsrc_b, dst + q_lo, HI ? loff_hi : loff_lo, HI ? toff_hi[0] : toff_lo[0], l_koff, l_tail);
+            dma_load_b128_select(IS_A ? rsrc_a : rsrc_b, dst + q_hi, HI ? loff_hi : loff_lo, HI ? toff_hi[1] : toff_lo[1],
+                                 l_koff + (uint32_t)(STREAM_SEGK * 2), l_tail);
+        } else {
+            dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_lo, HI ? loff_hi : loff_lo, l_koff);
+            dma_load_b128(IS_A ? rsrc_a : rsrc_b, dst + q_hi, HI ? loff_hi : loff_lo, l_koff + (uint32_t)(STREAM_SEGK * 2));
+        }
     };
 
     // ---- multiplier --------------------------------------------------------------------------------

@@ -9,9 +9,8 @@
  *   - a trailing `stream` (a hipStream_t passed as void*, NULL = default stream) is added;
  *   - "warps" are 64-lane wavefronts and "SMs" are compute units.
  * All pointers are device memory owned by the caller. Nothing is synchronised; launches are asynchronous on `stream`.
- * Device memory beyond the operands is needed in two cases only (zero-padded operand copies when K % 8 != 0, or
- * K % 64 != 0 with the straight-line kernel's tuple, or an operand is off a 16-byte boundary; partial planes when the
- * straight-line kernel cuts K into slices). The reference's
+ * Device memory beyond the operands is needed in two cases only (zero-padded operand copies when K % 8 != 0 or an
+ * operand is off a 16-byte boundary; partial planes when the straight-line kernel cuts K into slices). The reference's
  * launcher needs none and allocates nothing (port_2.cu:1088-1168; its drivers own all memory, :1200-1203). Here the
  * plain entry points take it from stream-ordered allocations on `stream` (hipMallocAsync / hipFreeAsync);
  * ckopt_gemm_shmem_tc_async_opt_port_2_ws takes it from a workspace the caller owns and allocates nothing;
@@ -54,10 +53,10 @@ enum {
  * reference's first tensor-core kernel, matmul_shmem_tc.cu:105-231); num_consumer_waves in {4,8}; num_cus = persistent grid.
  * M, N need not be multiples of tile_dim and K need not be a multiple of segment_dim_k (edges are
  * zero-filled / masked). The kernels read operand rows that start on 16-byte boundaries: when K is
- * not a multiple of 8 (of 64 for the tuple tile_dim 256, segment_dim_k 32, num_stages 5, no producer waves, whose
- * straight-line kernel works in whole loop bodies of 64), or A / Bt is not 16-byte aligned (2-byte alignment is
- * required), the call first copies both operands into zero-padded rows in a stream-ordered temporary
- * (hipMallocAsync / hipFreeAsync on `stream`, (M + N) * round_up(K, 8 or 64) * 2 bytes). */
+ * not a multiple of 8, or A / Bt is not 16-byte aligned (2-byte alignment is required), the call first copies both
+ * operands into zero-padded rows in a stream-ordered temporary (hipMallocAsync / hipFreeAsync on `stream`,
+ * (M + N) * Kp * 2 bytes with Kp = round_up(K, 8), or round_up(K, 64) for the tuple tile_dim 256, segment_dim_k 32,
+ * num_stages 5, no producer waves, whose straight-line kernel works in loop bodies of 64). */
 int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* Bt, const float* C, float* D,
                                          float alpha, float beta, int M, int N, int K, int tile_dim,
                                          int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
@@ -94,8 +93,8 @@ int ckopt_gemm_shmem_tc_async_opt_port_2_ws(int dtype, int cd_dtype, const void*
 /* The port_2 launcher above for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference, whose launcher needs no
  * memory beyond its operands. Same parameters and results as ckopt_gemm_shmem_tc_async_opt_port_2 (the same kernels
- * in the same order), but the zero-padded operand copies (K % 8 != 0, K % 64 != 0 with the straight-line tuple, or
- * operands off a 16-byte boundary: (M + N) * round_up(K, 8 or 64) * 2 bytes) and the split-K planes (slices * M * N * 4 bytes) live in a static device array
+ * in the same order), but the zero-padded operand copies (K % 8 != 0 or operands off a 16-byte boundary:
+ * (M + N) * round_up(K, 8 or 64) * 2 bytes) and the split-K planes (slices * M * N * 4 bytes) live in a static device array
  * of CKOPT_NOALLOC_SCRATCH_BYTES inside the library instead of stream-ordered allocations: no hipMalloc, hipFree or
  * allocating library routine is called. A launch that needs more than the array holds (both pieces, each rounded up
  * to 256 bytes) returns CKOPT_ERR_TOO_LARGE and D is not written; ckopt_set_option(7, 0) makes such a launch
@@ -185,9 +184,9 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  *        consumer bursts per SIMD pair, 2 none); key 4: producers' polling nap (0, 1, 2 = s_sleep 1, 4, 16);
  * key 5: tile granularity with dedicated producers synchronises through the hardware workgroup barrier
  *        (gemm_pcb_kernel, needs num_stages >= 2) instead of LDS counters (default 0).
- * key 6: launches with num_producer_warps 0, tile_dim 256, segment_dim_k 32, num_stages 5, 8 consumer warps (any M, N;
- *        K that is not a multiple of 64 is zero-padded to one in the operand copies) take the straight-line kernel
- *        written for exactly that shape (gemm_stream_kernel; default 1); 0 sends them through the general fused kernel.
+ * key 6: launches with num_producer_warps 0, tile_dim 256, segment_dim_k 32, num_stages 5, 8 consumer warps (any M, N, K)
+ *        take the straight-line kernel written for exactly that shape (gemm_stream_kernel; default 1); 0 sends them
+ *        through the general fused kernel.
  * key 7: split-K of the straight-line kernel. 1 (default): when a launch has fewer tiles than half the CUs (a
  *        multiple of 32 of them, or fewer than 32; N % 4 == 0) and K allows at least four slices of at least 1024
  *        that are multiples of 64, K is cut into num_sms / tiles slices (at most 16); the slices' partial products

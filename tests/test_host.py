@@ -228,7 +228,7 @@ def test_suggested_tunings_are_legal_and_follow_the_measured_rules(ck):
     assert picks(1024, 1024, 8192) == straight          # 16 tiles, eight slices of 1024
     assert picks(2048, 2048, 2048)["tile_dim"] == 128   # 64 tiles of 256 and K too shallow to cut four times
     assert picks(512, 512, 512)["tile_dim"] == 64       # config 1
-    assert picks(8192, 8192, 8200) == straight          # any K: the operand copies pad it to whole loop bodies of 64
+    assert picks(8192, 8192, 8200) == straight          # any K: its end is masked in the kernel (or in the operand copies)
     prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
     try:
         assert picks(8192, 8192, 8192)["num_producer_warps"] == 2 and picks(8192, 8192, 8192)["tile_dim"] == 256
@@ -287,9 +287,11 @@ def test_workspace_query_follows_the_launcher_rules(ck):
     assert ck.gemm_workspace_bytes(256, 256, 32768, True, *pc) == 0
     # copies and planes together (2 x 3 tiles, K 4090 -> 4096, four slices)
     assert ck.gemm_workspace_bytes(300, 520, 4090, True, *straight) == r256((300 + 520) * 4096 * 2) + r256(4 * 300 * 520 * 4) + 256
-    # K 8200 with the straight-line tuple: copies with rows of 8256 (whole loop bodies of 64); other tuples need none
-    assert ck.gemm_workspace_bytes(8192, 8192, 8200, True, *straight) == r256(2 * 8192 * 8256 * 2) + 256
-    assert ck.gemm_workspace_bytes(8192, 8192, 8200, True, *pc) == 0
+    # K 8200 (a multiple of 8): no copies, the straight-line kernel masks the end of K itself; K 8201: copies, with rows
+    # of 8256 (whole loop bodies of 64) for the straight-line tuple and of 8208 for the others
+    assert ck.gemm_workspace_bytes(8192, 8192, 8200, True, *straight) == 0
+    assert ck.gemm_workspace_bytes(8192, 8192, 8201, True, *straight) == r256(2 * 8192 * 8256 * 2) + 256
+    assert ck.gemm_workspace_bytes(8192, 8192, 8201, True, *pc) == r256(2 * 8192 * 8208 * 2) + 256
     # the split-K switch is part of the rule
     prev = ck.set_option(ck.OPT_SPLIT_K, 0)
     try:
