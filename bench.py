@@ -441,14 +441,22 @@ def main():
         # what the bare inner loop of this tile shape sustains on this device with random operands and the
         # loads of the real data flow (no synchronisation, no waiting, no epilogue): the device's power limit
         # keeps it well below the nominal peak, and no kernel of this shape can exceed it
-        ceil = mfma_ceiling(1, 1, 400000)
-        out["roofline"]["measured_ceiling"] = round(ceil, 1)
-        out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
+        try:   # a measurement aid in its own library: without it the line is printed without the ceiling
+            ceil = mfma_ceiling(1, 1, 400000)
+            out["roofline"]["measured_ceiling"] = round(ceil, 1)
+            out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
+        except (RuntimeError, OSError) as e:
+            out["roofline"]["measured_ceiling"] = None
+            print("ceiling probe not run: %s" % e, file=sys.stderr)
     if kind == "simt" and not args.no_ceiling:
         # the same for the vector ALUs: the micro-tile's multiply-add stream with random operands and nothing to feed it
-        ceil = valu_ceiling(1)
-        out["roofline"]["measured_ceiling"] = round(ceil, 1)
-        out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
+        try:
+            ceil = valu_ceiling(1)
+            out["roofline"]["measured_ceiling"] = round(ceil, 1)
+            out["roofline"]["frac_of_measured_ceiling"] = round(achieved / ceil, 4)
+        except (RuntimeError, OSError) as e:
+            out["roofline"]["measured_ceiling"] = None
+            print("ceiling probe not run: %s" % e, file=sys.stderr)
     if kind == "gemm" and args.workload == "config3_fp16_8192" and not args.no_vendor:
         # for orientation, outside the timed region: the vendor library's kernel for the same product on the same operands
         # (fp16 in, fp32 out), timed the same way right after ours, i.e. at the same sustained clock
