@@ -220,11 +220,10 @@ int persistent_grid(int64_t tiles, int num_cus, int num_xcd, bool even_rounds) {
 
 // Number of K slices the straight-line kernel uses for `tiles` 256 x 256 tiles (1: no split). policy 0: never;
 // 1: automatic - fewer tiles than half the CUs and at least four legal slices (two gain less than the
-// reduction pass costs); >= 2: that many slices if legal, else the next smaller legal count. Legal: whole XCD
-// rounds of tiles (a multiple of 32, or fewer than 32), N % 4 == 0 (vector stores of the partial planes), slices
-// of whole loop bodies and at least SPLIT_K_MIN_SLICE deep.
-int split_k_slices(int64_t tiles, int N, int K, int num_cus, int policy) {
-    if (policy == 0 || !(tiles % 32 == 0 || tiles < 32) || N % 4 != 0) return 1;
+// reduction pass costs); >= 2: that many slices if legal, else the next smaller legal count. Legal: slices
+// of whole loop bodies and at least SPLIT_K_MIN_SLICE deep (any tile count, any N).
+int split_k_slices(int64_t tiles, int K, int num_cus, int policy) {
+    if (policy == 0 || tiles <= 0) return 1;
     int cand = policy >= 2 ? policy : (int)(num_cus / tiles);
     if (cand > 16) cand = 16;
     while (cand >= 2 && !(K % (cand * ck::STREAM_K_MULTIPLE_HOST) == 0 && K / cand >= SPLIT_K_MIN_SLICE)) --cand;
@@ -258,7 +257,7 @@ size_t scratch_need(int M, int N, int K, bool operands_aligned, const ck::GemmTu
     }
     if (straight_line_tuple(t)) {
         const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-        const int slices = split_k_slices(tiles, N, k, t.num_cus, g_split_k.load());
+        const int slices = split_k_slices(tiles, k, t.num_cus, g_split_k.load());
         if (slices > 1) need += scratch_round((size_t)slices * M * N * sizeof(float));
     }
     return need;
@@ -344,7 +343,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         // Few tiles and a deep K: cut K into slices so that every CU has an item, partial products into
         // a stream-ordered workspace, one reduction pass.
         const bool bek = g_barrier_every_kstep.load() != 0;
-        int slices = split_k_slices(tiles, N, K, t.num_cus, g_split_k.load());
+        int slices = split_k_slices(tiles, K, t.num_cus, g_split_k.load());
         const long long count = (long long)M * N;
         float* ws = nullptr;
         if (slices > 1) {
@@ -359,7 +358,9 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         } else {
             GemmArgs p = a;
             p.split_k = slices;
-            p.split_chunk = tiles < 32 ? (int)tiles : 32;
+            // items are dealt slice by slice in runs of split_chunk tiles: 32 (what an XCD runs at a time) when the tiles
+            // come in whole runs of 32, otherwise all tiles of a slice in one run
+            p.split_chunk = tiles % 32 == 0 ? 32 : (int)tiles;
             p.D = ws; p.C = nullptr; p.alpha = 1.f; p.beta = 0.f; p.out16 = 0; p.vec_store = 1;
             const int64_t items = tiles * slices;
             const int pgrid = (int)(items < t.num_cus ? items : t.num_cus);
@@ -542,7 +543,7 @@ int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out)
     static const int pc_256[10] = {256, 64, 0, 0, 256, 256, 4, 2, 2, 8};
     const int* pick = fused_64;
     const int64_t t256 = tiles(256);
-    const bool split_ok = split_k_slices(t256, N, kp, num_cus, g_split_k.load()) > 1;
+    const bool split_ok = split_k_slices(t256, kp, num_cus, g_split_k.load()) > 1;
     if (t256 * 2 >= num_cus) pick = g_straight_line.load() && g_swizzle.load() ? straight_line : pc_256;
     else if (split_ok && g_straight_line.load() && g_swizzle.load()) pick = straight_line;
     else if (tiles(128) * 2 >= num_cus) pick = fused_128;

@@ -710,6 +710,9 @@ def test_straight_line_kernel_headline_size_properties(ck):
     (2000, 1020, 4096, 4, 256, "f16"),    # ragged tiles
     (512, 768, 8192, 1, 256, "f16"),      # 6 tiles: fewer than one XCD round, automatic slicing (8 slices)
     (700, 300, 4096, 3, 4, "bf16"),       # 6 ragged tiles on 4 workgroups; 3 slices asked, 4096 has no 3 whole ones: 2
+    (1536, 1536, 8192, 1, 256, "f16"),    # 36 tiles (neither fewer than 32 nor whole runs of 32): automatic, 4 slices
+    (700, 301, 8192, 4, 256, "bf16"),     # N not a multiple of 4: rows of the planes and of D on 4-byte boundaries
+    (2048, 1100, 4096, 2, 7, "f16"),      # 40 tiles, two slices, seven workgroups
 ])
 def test_split_k_bit_exact(ck, M, N, K, slices, cus, dt_name):
     dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16

@@ -292,6 +292,8 @@ def test_workspace_query_follows_the_launcher_rules(ck):
     assert ck.gemm_workspace_bytes(8192, 8192, 8200, True, *straight) == 0
     assert ck.gemm_workspace_bytes(8192, 8192, 8201, True, *straight) == r256(2 * 8192 * 8256 * 2) + 256
     assert ck.gemm_workspace_bytes(8192, 8192, 8201, True, *pc) == r256(2 * 8192 * 8208 * 2) + 256
+    # 36 tiles (1536^2) with a deep K are cut as well: four slices
+    assert ck.gemm_workspace_bytes(1536, 1536, 8192, True, *straight) == 4 * 1536 * 1536 * 4 + 256
     # the split-K switch is part of the rule
     prev = ck.set_option(ck.OPT_SPLIT_K, 0)
     try:
