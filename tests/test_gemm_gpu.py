@@ -942,3 +942,73 @@ def test_workspace_query_and_launches_that_need_none(ck):
     assert np.array_equal(d.cpu().numpy(), (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32))
     with pytest.raises(ck.CkoptError):
         ck.gemm_workspace_bytes(M, N, K, True, 100, *order[1:])
+
+
+def test_random_tunings_entry_points_and_options_exact(ck):
+    # seeded sweep over every kernel design, synchronisation granularity, grid size, the process-wide options and the
+    # three homes of the scratch memory (stream-ordered allocation, caller's workspace, the library's static array):
+    # exact on small integers whatever the summation order; D starts out as NaN, so every element must be written
+    rng = np.random.default_rng(20251126)
+    ran = 0
+    for case in range(260):
+        if rng.random() < 0.35:
+            t = G.tuning(tile_dim=256, segment_dim_k=32, num_stages=5, num_producer_warps=0, num_consumer_warps=8,
+                         tile_group_m=int(rng.integers(1, 7)), num_sms=int(rng.choice([1, 3, 8, 40, 256])))
+        else:
+            tile = int(rng.choice([64, 128, 256]))
+            cw = 8 if tile == 256 else int(rng.choice([4, 8]))
+            p = int(rng.choice([0, 0, 2, 4, 8]))
+            t = G.tuning(tile_dim=tile, segment_dim_k=int(rng.choice([32, 64, 128])), num_stages=int(rng.integers(1, 6)),
+                         num_producer_warps=p, num_consumer_warps=cw, tile_group_m=int(rng.integers(1, 7)),
+                         num_sms=int(rng.choice([1, 3, 8, 40, 256])))
+            mode = "tile" if p == 0 else str(rng.choice(["tile", "wave", "acc"]))
+            wtr = ck.get_warp_tile_rows(tile, cw)
+            wtc = ck.get_num_acc(tile, cw) // wtr
+            if mode == "wave":
+                t["bar_step_rows_a"], t["bar_step_rows_b"] = wtr * 16, wtc * 16
+                t["bar_steps_a"], t["bar_steps_b"] = int(rng.integers(0, cw // 2 + 1)), int(rng.integers(0, 3))
+            elif mode == "acc":
+                t["bar_step_rows_a"] = t["bar_step_rows_b"] = 16
+                t["bar_steps_a"], t["bar_steps_b"] = int(rng.integers(0, wtr)), int(rng.integers(0, wtc))
+        order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b",
+                                "tile_group_m", "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
+        M, N = int(rng.integers(1, 700)), int(rng.integers(1, 700))
+        K = int(rng.choice([int(rng.integers(1, 1500)), 8 * int(rng.integers(1, 200)), 64 * int(rng.integers(1, 40)), 1024 * int(rng.integers(1, 7))]))
+        dt = ck.DT_F16 if rng.random() < 0.5 else ck.DT_BF16
+        alpha, beta = float(rng.choice([1.0, 2.0, -0.5])), float(rng.choice([0.0, 0.0, -1.0, 2.0]))
+        opts = {ck.OPT_SPLIT_K: int(rng.choice([0, 1, 1, 2, 3, 4, 8])), ck.OPT_BARRIER_EVERY_KSTEP: int(rng.integers(0, 2)),
+                ck.OPT_EVEN_ROUNDS: int(rng.integers(0, 2)), ck.OPT_TILE_SYNC_BARRIER: int(rng.integers(0, 2))}
+        entry = int(rng.integers(0, 3))
+        if ck.check_gemm_tuning(*order) != ck.OK:
+            continue
+        a = ck.fill_int(dt, (M, K), 3000 + case, 0, -2, 2)
+        bt = ck.fill_int(dt, (N, K), 3000 + case, 1, -2, 2)
+        c = ck.fill_int(ck.DT_F32, (M, N), 3000 + case, 2, -3, 3) if beta else None
+        want = alpha * (G.as_f64(dt == ck.DT_BF16, a) @ G.as_f64(dt == ck.DT_BF16, bt).T)
+        if beta:
+            want = want + beta * c.astype(np.float64)
+        prev = {k: ck.set_option(k, v) for k, v in opts.items()}
+        try:
+            da, db = G.to_dev(a), G.to_dev(bt)
+            dc = None if c is None else G.to_dev(c)
+            dd = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            try:
+                if entry == 0:
+                    ck.gemm_shmem_tc_async_opt_port(dt, da, db, dc, dd, alpha, beta, M, N, K, *order)
+                elif entry == 1:
+                    need = ck.gemm_workspace_bytes(M, N, K, True, *order)
+                    ws = torch.empty(need + 64, dtype=torch.uint8, device="cuda")
+                    ck.gemm_shmem_tc_async_opt_port_ws(dt, ck.DT_F32, da, db, dc, dd, alpha, beta, M, N, K, *order,
+                                                       ws.data_ptr() + int(rng.integers(0, 48)), need)
+                else:
+                    ck.gemm_shmem_tc_async_opt_port_noalloc(dt, da, db, dc, dd, alpha, beta, M, N, K, *order)
+            except ck.CkoptError as e:
+                assert e.code == ck.ERR_NO_INSTANCE, (case, order, e)
+                continue
+            assert ck.device_status() == 0
+            assert np.array_equal(dd.cpu().numpy(), want.astype(np.float32)), (case, (M, N, K), dt, alpha, beta, order, opts, entry)
+            ran += 1
+        finally:
+            for k, v in prev.items():
+                ck.set_option(k, v)
+    assert ran >= 150
