@@ -52,6 +52,8 @@ std::atomic<int> g_straight_line{1};
 std::atomic<int> g_even_rounds{1};
 std::atomic<int> g_split_k{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
 std::atomic<int> g_barrier_every_kstep{1};
+std::atomic<int> g_d_store_policy{0};  // 0: non-temporal stores of D where its rows lie on 128-byte lines, 1: always, 2: never
+constexpr int LINE_BYTES = 128;         // cache line of the vector memory path
 constexpr int SPLIT_K_MIN_SLICE = 1024;  // shortest K slice split-K will make (shorter ones lose more in the reduction pass than they gain)
 
 constexpr int MAX_DEV = 64;
@@ -324,6 +326,11 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     // one vector access per accumulator block: 16 bytes of fp32 need only the 4-byte alignment checked above
     // (any N); 8 bytes of 16-bit results need their own alignment
     a.vec_store = !out16 || ((N % 4 == 0) && !((uintptr_t)D & 7) && (beta == 0.f || !((uintptr_t)C & 7)));
+    // Non-temporal stores of D pay where the stores of a row fill whole 128-byte lines; rows that start anywhere make
+    // every 128-byte run straddle two lines, and only ordinary stores let the two parts meet in L2.
+    const int store_policy = g_d_store_policy.load();
+    auto whole_lines = [](const void* base, int64_t row_bytes) { return (uintptr_t)base % LINE_BYTES == 0 && row_bytes % LINE_BYTES == 0; };
+    a.nt_store = store_policy == 1 || (store_policy == 0 && whole_lines(D, (int64_t)N * (out16 ? 2 : 4)));
     a.spin_limit = (uint32_t)g_spin_limit.load();
     a.prio_mode = g_prio_mode.load();
     a.producer_nap = g_producer_nap.load();
@@ -362,6 +369,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             // come in whole runs of 32, otherwise all tiles of a slice in one run
             p.split_chunk = tiles % 32 == 0 ? 32 : (int)tiles;
             p.D = ws; p.C = nullptr; p.alpha = 1.f; p.beta = 0.f; p.out16 = 0; p.vec_store = 1;
+            p.nt_store = store_policy == 1 || (store_policy == 0 && whole_lines(ws, (int64_t)N * 4) && count * 4 % LINE_BYTES == 0);
             const int64_t items = tiles * slices;
             const int pgrid = (int)(items < t.num_cus ? items : t.num_cus);
             e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p, bek) : launch_gemm_stream_bf16(dim3(pgrid), s, p, bek);
@@ -621,6 +629,7 @@ int ckopt_set_option(int key, int value) {
         case 7: if (value < 0 || value > 16) return ck::CK_ERR_BAD_PARAM; return g_split_k.exchange(value);
         case 8: return g_barrier_every_kstep.exchange(value != 0);
         case 9: return g_even_rounds.exchange(value != 0);
+        case 10: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_d_store_policy.exchange(value);
         default: return ck::CK_ERR_BAD_PARAM;
     }
 }

@@ -63,6 +63,8 @@ struct GemmArgs {
     int num_xcd;
     int vec_store;  // C and D allow one vector access per accumulator block (fp32: always; 16-bit: N % 4 == 0, 8-byte aligned)
     int out16;      // C and D hold the operands' 16-bit element type instead of fp32 (accumulation stays fp32)
+    int nt_store;   // D's rows start on 128-byte lines: vector stores of D are non-temporal (they fill whole lines and need not
+                    // stay in L2); otherwise ordinary stores, so that the two parts of a line written by different stores meet in L2
     int split_k;    // straight-line kernel only: K is cut into this many slices (>= 1), one work item per (tile, slice);
                     // slice s writes its partial products to D + s * M * N (a workspace; alpha 1, beta 0, fp32)
     int split_chunk;  // consecutive work items that belong to one slice (32 = one XCD round, or all tiles if fewer)
@@ -106,6 +108,14 @@ template <> struct Out16<bf16_tag> {
         return (unsigned short)(u >> 16);
     }
 };
+// Non-temporal vector stores, written as asm: as a compiler builtin in one branch of a run-time switch with an ordinary
+// store of the same value in the other, the two are merged into one ordinary store and the hint is lost. (Addresses
+// need 4-byte alignment only. The stores are not waited for anywhere; waits the compiler places for its own loads
+// only become stronger by stores it does not know of, since vector memory operations complete in issue order.)
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store_b128_nt(void* p, u32x4 v) { asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(p), "v"(v) : "memory"); }
+__device__ __forceinline__ void store_b64_nt(void* p, u32x2 v) { asm volatile("global_store_dwordx2 %0, %1, off nt" ::"v"(p), "v"(v) : "memory"); }
+
 // vec_cols: the tile's columns all lie inside the matrix and C / D allow one vector access per block (fp32: always;
 // 16-bit: N % 4 == 0 and 8-byte aligned pointers); rows past M are skipped. Otherwise element by element.
 template <typename DT>
@@ -118,7 +128,9 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
         if (vec_cols) {
             if (beta != 0.f) v += *(const f32x4_u*)(g.C + off) * beta;
             // D is written once and not read again: non-temporal, so that it does not displace the operands in L2
-            __builtin_nontemporal_store(v, (f32x4_u*)(g.D + off));
+            // (rows off the 128-byte lines: ordinary stores, whose partial lines are merged in L2 before they reach memory)
+            if (g.nt_store) store_b128_nt(g.D + off, __builtin_bit_cast(u32x4, v));
+            else *(f32x4_u*)(g.D + off) = v;
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -143,8 +155,8 @@ __device__ __forceinline__ void epilogue_block(const GemmArgs& g, int m, int n, 
             uint2 o;
             o.x = (uint32_t)Out16<DT>::store(v[0]) | ((uint32_t)Out16<DT>::store(v[1]) << 16);
             o.y = (uint32_t)Out16<DT>::store(v[2]) | ((uint32_t)Out16<DT>::store(v[3]) << 16);
-            typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-            __builtin_nontemporal_store(u32x2{o.x, o.y}, (u32x2*)(d16 + off));
+            if (g.nt_store) store_b64_nt(d16 + off, u32x2{o.x, o.y});
+            else *(u32x2*)(d16 + off) = u32x2{o.x, o.y};
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {

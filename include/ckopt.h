@@ -200,6 +200,11 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  *        persistent grid is the smallest number of workgroups (a multiple of the XCD count, at most num_sms) that
  *        needs no more rounds, so that no round is partly empty (408 tiles on 256 CUs: 208 workgroups x 2 rounds
  *        instead of 256 + 152; 5.7 % faster where the clock is power-limited); 0: always min(tiles, num_sms).
+ * key 10: how the GEMM kernels store D. 0 (default): non-temporal vector stores where every row of D starts on a 128-byte
+ *        line (D on a 128-byte boundary and N * element size a multiple of 128), ordinary stores otherwise: rows that
+ *        start anywhere make every 128-byte run of a row straddle two lines, and only ordinary stores let the parts
+ *        meet in L2 before they reach memory (bf16 6143 x 4097 x 3072: 138 us against 164). 1: always non-temporal;
+ *        2: never.
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

@@ -577,6 +577,46 @@ def test_straight_line_kernel_any_k(ck, M, N, K):
         assert ck.gemm_workspace_bytes(M, N, K, True, *order) == 0    # K % 64 != 0 is masked inside the kernel
 
 
+@pytest.mark.parametrize("N", [512, 516, 301])   # rows of D on 128-byte lines / on 16-byte boundaries only / anywhere
+def test_d_store_policy_exact(ck, N):
+    """Non-temporal and ordinary stores of D (the launcher chooses by the alignment of D's rows; the option forces
+    either): same exact small-integer results from the straight-line kernel, a general kernel, split-K planes and the
+    16-bit epilogues, whole matrix, every element written (D starts as NaN)."""
+    M, K = 520, 2048
+    for dt in (ck.DT_F16, ck.DT_BF16):
+        is_bf = dt == ck.DT_BF16
+        a = ck.fill_int(dt, (M, K), 55, 0, -1, 1)
+        bt = ck.fill_int(dt, (N, K), 55, 1, -1, 1)
+        c = ck.fill_int(ck.DT_F32, (M, N), 55, 2, -3, 3)
+        exact = G.as_f64(is_bf, a) @ G.as_f64(is_bf, bt).T
+        tdt = torch.bfloat16 if is_bf else torch.float16
+        for policy in (0, 1, 2):
+            prev = ck.set_option(ck.OPT_D_STORE_POLICY, policy)
+            try:
+                for t in (_straight_line_tuning(ck), make_tuning(ck, 128, 64, 2, 2, 8), make_tuning(ck, 128, 64, 2, 0, 4)):
+                    assert np.array_equal(G.run_gemm(ck, dt, a, bt, t=t), exact.astype(np.float32)), (policy, t)
+                    assert np.array_equal(G.run_gemm(ck, dt, a, bt, c, -1.0, 2.0, t=t), (2.0 * c - exact).astype(np.float32)), (policy, t)
+                before = ck.set_option(ck.OPT_SPLIT_K, 2)   # K = 2048: two slices of 1024 through the planes
+                try:
+                    assert np.array_equal(G.run_gemm(ck, dt, a, bt, t=_straight_line_tuning(ck)), exact.astype(np.float32)), policy
+                finally:
+                    ck.set_option(ck.OPT_SPLIT_K, before)
+                # 16-bit C and D (|sums| stay far below 2048, so every result is representable)
+                small = exact[:, :] * 0.0625
+                for t in (_straight_line_tuning(ck), make_tuning(ck, 128, 64, 2, 2, 8)):
+                    da, db = G.to_dev(a), G.to_dev(bt)
+                    dd = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+                    ck.gemm_shmem_tc_async_opt_port_lp(dt, da, db, None, dd, 0.0625, 0.0, M, N, K, t["tile_dim"], t["segment_dim_k"],
+                                                       t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                                       t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                                       t["num_consumer_warps"], t["num_sms"])
+                    assert ck.device_status() == 0
+                    want16 = torch.from_numpy(small.astype(np.float32)).to(tdt).float().numpy()
+                    assert np.array_equal(dd.float().cpu().numpy(), want16), (policy, t)
+            finally:
+                ck.set_option(ck.OPT_D_STORE_POLICY, prev)
+
+
 @pytest.mark.parametrize("M,N,K,cus", [
     (1280, 1280, 192, 24),   # 25 tiles on 24 workgroups: 2 rounds, even rounds take 16 workgroups
     (1279, 1025, 320, 12),   # ragged, 25 tiles on 12: 3 rounds, 9 -> 12 workgroups (rounded up to whole XCDs, capped)

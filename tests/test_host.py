@@ -198,7 +198,7 @@ def test_normal_and_int_generators(ck):
 
 def test_option_keys_reject_values_outside_their_range(ck):
     # process-wide switches: a bad value changes nothing and reports the error
-    for key, bad in ((ck.OPT_NUM_XCD, 0), (ck.OPT_PRIO_MODE, 3), (ck.OPT_PRODUCER_NAP, -1), (ck.OPT_SPLIT_K, 17), (99, 1)):
+    for key, bad in ((ck.OPT_NUM_XCD, 0), (ck.OPT_PRIO_MODE, 3), (ck.OPT_PRODUCER_NAP, -1), (ck.OPT_SPLIT_K, 17), (ck.OPT_D_STORE_POLICY, 3), (99, 1)):
         with pytest.raises(ck.CkoptError):
             ck.set_option(key, bad)
     prev = ck.set_option(ck.OPT_SPLIT_K, 0)
@@ -207,6 +207,8 @@ def test_option_keys_reject_values_outside_their_range(ck):
     assert ck.set_option(ck.OPT_STRAIGHT_LINE, prev) == 0
     prev = ck.set_option(ck.OPT_EVEN_ROUNDS, 0)
     assert prev == 1 and ck.set_option(ck.OPT_EVEN_ROUNDS, prev) == 0
+    prev = ck.set_option(ck.OPT_D_STORE_POLICY, 2)
+    assert prev == 0 and ck.set_option(ck.OPT_D_STORE_POLICY, prev) == 2
 
 
 def test_suggested_tunings_are_legal_and_follow_the_measured_rules(ck):
