@@ -93,7 +93,7 @@ int static_scratch_for_current_device(unsigned char** out) {
 
 // Copies `rows` rows of K 2-byte elements into rows of Kp >= K elements (Kp % 8 == 0), zero filling
 // the tail: the form the direct-to-LDS loads need (every row starts on a 16-byte boundary). One
-// thread produces one 16-byte chunk of the destination from eight 2-byte reads.
+// thread produces one 16-byte chunk of the destination.
 // Both operands go through one launch: chunks [0, rows_a * Kp / 8) belong to A, the rest to Bt.
 __global__ void pad_rows_kernel(const unsigned short* __restrict__ src_a, unsigned short* __restrict__ dst_a, int rows_a,
                                 const unsigned short* __restrict__ src_b, unsigned short* __restrict__ dst_b, int rows_b, int K, int Kp) {
@@ -106,7 +106,14 @@ __global__ void pad_rows_kernel(const unsigned short* __restrict__ src_a, unsign
         unsigned short* dst = second ? dst_b : dst_a;
         const long long c = second ? cc - total_a : cc;
         const int r = (int)(c / chunks_per_row), k0 = (int)(c % chunks_per_row) * 8;
-        // The chunk's 16 source bytes start on a 2-byte boundary: five aligned 4-byte words cover them,
+        if (k0 + 8 <= K) {
+            // a whole chunk of the row: one 16-byte load (the vector memory path takes 2-byte-aligned addresses)
+            typedef unsigned int u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+            const u32x4_a2 v = *reinterpret_cast<const u32x4_a2*>(src + (long long)r * K + k0);
+            *reinterpret_cast<uint4*>(dst + (long long)r * Kp + k0) = uint4{v[0], v[1], v[2], v[3]};
+            continue;
+        }
+        // The chunk that holds the end of the row (or lies past it). Its 16 source bytes start on a 2-byte boundary: five aligned 4-byte words cover them,
         // shifted by two bytes where the start is odd. A word that lies only half inside
         // [chunk start, row end) is read as that one element, so no byte outside the row is touched.
         const uintptr_t first = (uintptr_t)(src + (long long)r * K + k0);
