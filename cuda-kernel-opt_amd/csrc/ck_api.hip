@@ -1,7 +1,9 @@
 // extern "C" launch layer: parameter validation, instance dispatch, device status word.
 // Declarations and the reference launcher each entry point replaces are in include/ckopt.h.
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <atomic>
+#include <cmath>
 #include <mutex>
 #include <type_traits>
 
@@ -227,18 +229,45 @@ int persistent_grid(int64_t tiles, int num_cus, int num_xcd, bool even_rounds) {
     return (int)(g < num_cus ? g : num_cus);
 }
 
+// Estimated duration (microseconds) of the straight-line kernel on `tiles` 256 x 256 tiles of an M x N product with K cut
+// into S slices, plus the reduction pass when S > 1. The constants are measurements of one MI355X on random operands:
+// a loop body (64 of K) takes 1.05 us while at most half of the 256 CUs multiply and the clock is free, and grows with
+// the number of active CUs once the device is power-limited (1.42 us with all of them); a work item costs about 3 us
+// of pipeline fill and drain; the items of a round store their 256 KiB each at the 4.6 TB/s the write path sustains;
+// the reduction pass reads S planes and writes D at 5.3 TB/s behind about 3 us of launch.
+double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus) {
+    const double items = (double)tiles * S;
+    const double rounds = std::ceil(items / num_cus);
+    const double active = items / rounds;   // workgroups (CUs) busy in a round
+    const double body_us = 1.05 * std::max(1.0, std::pow(active / 128.0, 0.43));
+    const double bodies = (double)K / S / ck::STREAM_K_MULTIPLE_HOST;
+    const double store_us = active * (256.0 * 1024.0) / 4.6e6;
+    double t = rounds * (bodies * body_us + store_us + 3.0);
+    if (S > 1) t += 3.0 + (double)(S + 1) * (double)mn * 4.0 / 5.3e6;
+    return t;
+}
+
 // Number of K slices the straight-line kernel uses for `tiles` 256 x 256 tiles (1: no split). policy 0: never;
-// 1: automatic - fewer tiles than half the CUs and at least four legal slices (two gain less than the
-// reduction pass costs); >= 2: that many slices if legal, else the next smaller legal count. Legal: slices
-// of whole loop bodies and at least SPLIT_K_MIN_SLICE deep (any tile count, any N).
-int split_k_slices(int64_t tiles, int K, int num_cus, int policy) {
+// 1: automatic - with fewer tiles than CUs, the legal slice count whose estimated duration is shortest (a larger count
+// must win by 3 %: it costs scratch memory); >= 2: that many slices if legal, else the next smaller legal count.
+// Legal: slices of whole loop bodies and at least SPLIT_K_MIN_SLICE deep (any tile count, any N).
+int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, int policy) {
     if (policy == 0 || tiles <= 0) return 1;
-    int cand = policy >= 2 ? policy : (int)(num_cus / tiles);
-    if (cand > 16) cand = 16;
-    while (cand >= 2 && !(K % (cand * ck::STREAM_K_MULTIPLE_HOST) == 0 && K / cand >= SPLIT_K_MIN_SLICE)) --cand;
-    if (cand < 2) return 1;
-    if (policy >= 2) return cand;
-    return tiles * 2 <= num_cus && cand >= 4 ? cand : 1;
+    auto legal = [&](int c) { return K % (c * ck::STREAM_K_MULTIPLE_HOST) == 0 && K / c >= SPLIT_K_MIN_SLICE; };
+    if (policy >= 2) {
+        int cand = policy > 16 ? 16 : policy;
+        while (cand >= 2 && !legal(cand)) --cand;
+        return cand < 2 ? 1 : cand;
+    }
+    if (tiles >= num_cus) return 1;
+    int best = 1;
+    double best_us = split_k_estimate_us(tiles, mn, K, 1, num_cus);
+    for (int c = 2; c <= 16; ++c) {
+        if (!legal(c)) continue;
+        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus);
+        if (us < 0.97 * best_us) { best = c; best_us = us; }
+    }
+    return best;
 }
 
 // The tuning tuple the straight-line kernel is written for (it also needs K in whole loop bodies of 64).
@@ -266,7 +295,7 @@ size_t scratch_need(int M, int N, int K, bool operands_aligned, const ck::GemmTu
     }
     if (straight_line_tuple(t)) {
         const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-        const int slices = split_k_slices(tiles, k, t.num_cus, g_split_k.load());
+        const int slices = split_k_slices(tiles, (int64_t)M * N, k, t.num_cus, g_split_k.load());
         if (slices > 1) need += scratch_round((size_t)slices * M * N * sizeof(float));
     }
     return need;
@@ -357,7 +386,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         // Few tiles and a deep K: cut K into slices so that every CU has an item, partial products into
         // a stream-ordered workspace, one reduction pass.
         const bool bek = g_barrier_every_kstep.load() != 0;
-        int slices = split_k_slices(tiles, K, t.num_cus, g_split_k.load());
+        int slices = split_k_slices(tiles, (int64_t)M * N, K, t.num_cus, g_split_k.load());
         const long long count = (long long)M * N;
         float* ws = nullptr;
         if (slices > 1) {
@@ -558,7 +587,7 @@ int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out)
     static const int pc_256[10] = {256, 64, 0, 0, 256, 256, 4, 2, 2, 8};
     const int* pick = fused_64;
     const int64_t t256 = tiles(256);
-    const bool split_ok = split_k_slices(t256, kp, num_cus, g_split_k.load()) > 1;
+    const bool split_ok = split_k_slices(t256, (int64_t)M * N, kp, num_cus, g_split_k.load()) > 1;
     if (t256 * 2 >= num_cus) pick = g_straight_line.load() && g_swizzle.load() ? straight_line : pc_256;
     else if (split_ok && g_straight_line.load() && g_swizzle.load()) pick = straight_line;
     else if (tiles(128) * 2 >= num_cus) pick = fused_128;

@@ -187,11 +187,12 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  * key 6: launches with num_producer_warps 0, tile_dim 256, segment_dim_k 32, num_stages 5, 8 consumer warps (any M, N, K)
  *        take the straight-line kernel written for exactly that shape (gemm_stream_kernel; default 1); 0 sends them
  *        through the general fused kernel.
- * key 7: split-K of the straight-line kernel. 1 (default): when a launch has fewer tiles than half the CUs and K allows
- *        at least four slices of at least 1024 that are multiples of 64, K is cut into num_sms / tiles slices (at
- *        most 16); the slices' partial products go to scratch memory (slices * M * N * 4 bytes) and a second kernel
- *        adds them in slice order and applies alpha, beta and the output type. 0: never. 2..16: that many slices
- *        whenever legal.
+ * key 7: split-K of the straight-line kernel. 1 (default): with fewer tiles than num_sms, K is cut into the number of
+ *        slices (at most 16, each a multiple of 64 and at least 1024 deep) for which a cost model of the device gives
+ *        the shortest time - loop bodies at the rate the active CUs sustain, the store burst of every round, the
+ *        reduction pass (e.g. 64 tiles, K 32768: 4 slices; 128 tiles, K 16384: 2; 128 tiles, K 4096: none); the
+ *        slices' partial products go to scratch memory (slices * M * N * 4 bytes) and a second kernel adds them in
+ *        slice order and applies alpha, beta and the output type. 0: never. 2..16: that many slices whenever legal.
  * key 8: schedule of the straight-line kernel. 1 (default): a workgroup barrier in every k-step, the loads of a loop
  *        body spread over both (three k-steps to land); 0: one barrier per two k-steps, all loads behind it (two
  *        k-steps to land) - 1.5 % faster at 8192^3 on random operand values (power-limited clock), slower wherever

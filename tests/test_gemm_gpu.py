@@ -769,6 +769,19 @@ def test_split_k_bit_exact(ck, M, N, K, slices, cus, dt_name):
     assert np.array_equal(got, want)
 
 
+def test_automatic_split_k_of_128_tiles_exact(ck):
+    # 128 tiles on 256 CUs with a deep K: the automatic rule cuts K in two (256 work items); exact on small integers
+    M, N, K = 2048, 4096, 8192
+    t = _straight_line_tuning(ck)
+    order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b",
+                            "tile_group_m", "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
+    assert ck.gemm_workspace_bytes(M, N, K, True, *order) == 2 * M * N * 4 + 256
+    a = ck.fill_int(ck.DT_F16, (M, K), 97, 0, -1, 1)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 97, 1, -1, 1)
+    want = (a.astype(np.float32) @ bt.astype(np.float32).T)   # sums of at most 8192 terms of -1, 0, 1: exact in fp32
+    assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want)
+
+
 def test_split_k_against_the_oracle_and_the_single_pass(ck, oracle):
     # uniform data: the sliced sum differs from the single pass in rounding only
     M, N, K = 2048, 1024, 4096

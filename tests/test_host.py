@@ -296,6 +296,13 @@ def test_workspace_query_follows_the_launcher_rules(ck):
     assert ck.gemm_workspace_bytes(8192, 8192, 8201, True, *pc) == r256(2 * 8192 * 8208 * 2) + 256
     # 36 tiles (1536^2) with a deep K are cut as well: four slices
     assert ck.gemm_workspace_bytes(1536, 1536, 8192, True, *straight) == 4 * 1536 * 1536 * 4 + 256
+    # the automatic slice count follows the launcher's cost model: 128 tiles with a deep K are cut in two (256 items),
+    # with K 4096 not at all (the reduction pass would cost more than the idle half of the CUs); 81 tiles in three;
+    # 144 tiles never (two slices would be 288 items: two rounds)
+    assert ck.gemm_workspace_bytes(2048, 4096, 16384, True, *straight) == 2 * 2048 * 4096 * 4 + 256
+    assert ck.gemm_workspace_bytes(2048, 4096, 4096, True, *straight) == 0
+    assert ck.gemm_workspace_bytes(2304, 2304, 12288, True, *straight) == 3 * 2304 * 2304 * 4 + 256
+    assert ck.gemm_workspace_bytes(3072, 3072, 8192, True, *straight) == 0
     # the split-K switch is part of the rule
     prev = ck.set_option(ck.OPT_SPLIT_K, 0)
     try:
