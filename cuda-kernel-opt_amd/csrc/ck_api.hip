@@ -587,10 +587,22 @@ int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out)
     static const int pc_256[10] = {256, 64, 0, 0, 256, 256, 4, 2, 2, 8};
     const int* pick = fused_64;
     const int64_t t256 = tiles(256);
-    const bool split_ok = split_k_slices(t256, (int64_t)M * N, kp, num_cus, g_split_k.load()) > 1;
-    if (t256 * 2 >= num_cus) pick = g_straight_line.load() && g_swizzle.load() ? straight_line : pc_256;
-    else if (split_ok && g_straight_line.load() && g_swizzle.load()) pick = straight_line;
-    else if (tiles(128) * 2 >= num_cus) pick = fused_128;
+    const bool straight_ok = g_straight_line.load() && g_swizzle.load();
+    if (!straight_ok) {
+        // without the straight-line kernel: the reference's design on 256 tiles when they fill half the device
+        if (t256 * 2 >= num_cus) pick = pc_256;
+        else if (tiles(128) * 2 >= num_cus) pick = fused_128;
+    } else {
+        // the shortest of three estimates: the straight-line kernel with the slice count the launcher would choose
+        // (split_k_estimate_us), and the general kernel on 128 and on 64 tiles - one workgroup per CU, measured per
+        // 128 of K: 1.4 us for a 128 x 128 tile, 0.65 us for a 64 x 64 tile, about 4 us per round besides
+        const int slices = split_k_slices(t256, (int64_t)M * N, kp, num_cus, g_split_k.load());
+        const double straight_us = split_k_estimate_us(t256, (int64_t)M * N, kp, slices, num_cus);
+        auto general_us = [&](int t, double seg_us) { return std::ceil((double)tiles(t) / num_cus) * ((double)K / 128.0 * seg_us + 4.0); };
+        const double us_128 = general_us(128, 1.4), us_64 = general_us(64, 0.65);
+        if (straight_us <= us_128 && straight_us <= us_64) pick = straight_line;
+        else if (us_128 <= us_64) pick = fused_128;
+    }
     for (int i = 0; i < 10; ++i) tuning_out[i] = pick[i];
     return CK_OK;
 }
