@@ -179,6 +179,61 @@ def sweep(ck, torch, args, ckdt, da, db, dd, M, N, K, cus, stream):
     return 0
 
 
+GRID_SHAPES = [(512, 512, 512), (1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (2560, 2560, 2560), (3072, 3072, 3072), (4096, 4096, 4096),
+               (6144, 6144, 6144), (8192, 8192, 8192), (1024, 1024, 8192), (1024, 8192, 1024), (8192, 1024, 1024), (512, 8192, 8192), (8192, 8192, 512),
+               (8192, 8192, 1024), (256, 16384, 4096), (16384, 256, 4096), (4096, 4096, 256), (2048, 2048, 32768), (1024, 1024, 65536), (2048, 4096, 16384),
+               (2304, 2304, 12288), (6143, 4097, 3071), (5000, 5000, 5000), (3000, 7000, 2000), (8192, 4096, 2048), (12288, 4096, 4096), (4096, 11008, 4096),
+               (2048, 8192, 8192)]
+
+
+def grid(ck, torch, cus, stream):
+    """fp16 products of many shapes, each on the tuple the library suggests for it, with the vendor library's GEMM
+    (torch.mm, fp32 output) on the same operands beside it: one text line per shape, then one JSON line."""
+    def timeit(fn, flops):
+        n = max(10, int(0.02 / (flops / 1.0e15)))
+        for _ in range(max(20, n // 2)):
+            fn()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(2):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(n):
+                fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / n * 1e3
+            best = us if best is None else min(best, us)
+        return best
+    rows = []
+    for M, N, K in GRID_SHAPES:
+        a = ck.fill_uniform(ck.DT_F16, (M, K), 11, 0, -1.0, 1.0)
+        b = ck.fill_uniform(ck.DT_F16, (N, K), 11, 1, -1.0, 1.0)
+        da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+        dd = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        t = ck.suggest_gemm_tuning(M, N, K, cus)
+        tup = (t["tile_dim"], t["segment_dim_k"], t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"], t["tile_group_m"],
+               t["num_stages"], t["num_producer_warps"], t["num_consumer_warps"])
+        flops = 2.0 * M * N * K
+        ours = timeit(lambda: ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, da, db, None, dd, 1.0, 0.0, M, N, K, *tup, cus, stream), flops)
+        tb = db.t()
+        try:
+            vend = timeit(lambda: torch.mm(da, tb, out_dtype=torch.float32), flops)
+        except Exception:   # a torch without out_dtype
+            vend = None
+        if ck.device_status() != 0:
+            print("device status non-zero at %s" % ((M, N, K),), file=sys.stderr)
+            return 4
+        row = {"M": M, "N": N, "K": K, "tuple": list(tup), "us": round(ours, 1), "tflops": round(flops / ours * 1e-6, 1),
+               "vendor_us": None if vend is None else round(vend, 1), "vendor_tflops": None if vend is None else round(flops / vend * 1e-6, 1)}
+        rows.append(row)
+        print("%6d x %6d x %6d  (%s): %8.1f us %7.1f TFLOP/s | vendor library %s" % (
+            M, N, K, ", ".join(str(v) for v in tup), ours, row["tflops"],
+            "not timed" if vend is None else "%8.1f us %7.1f TFLOP/s, ours / vendor %.2f" % (vend, row["vendor_tflops"], vend / ours)), flush=True)
+    print(json.dumps({"grid": "fp16, uniform[-1,1), fp32 output; suggested tuple per shape; vendor = torch.mm(A, Bt.T, out_dtype=float32)", "rows": rows}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -214,6 +269,8 @@ def main():
                     help="skip timing the vendor library's GEMM (hipBLASLt through torch.mm, fp32 output) on the same operands")
     ap.add_argument("--no-settle", action="store_true",
                     help="skip the set-up launches that bring the device to its sustained clock before warm-up")
+    ap.add_argument("--grid", action="store_true",
+                    help="fp16 products of many shapes on the tuple the library suggests for each, with the vendor library's GEMM beside it")
     ap.add_argument("--sweep", action="store_true",
                     help="time a list of tuning tuples on the workload (the role of the reference drivers' performance "
                          "loops, port_2.cu:1463-1480): one line per tuple in the reference's format, then one JSON line")
@@ -259,6 +316,8 @@ def main():
         k, v = kv.split("=")
         ck.set_option(int(k), int(v))
         options[int(k)] = int(v)
+    if args.grid:
+        return grid(ck, torch, cus, torch.cuda.current_stream())
 
     kind, dtype, M, N, K, dist = WORKLOADS[args.workload]
     # tuning flags default to what the library suggests for the shape (ckopt_suggest_gemm_tuning); TUNED records
