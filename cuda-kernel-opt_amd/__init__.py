@@ -19,6 +19,7 @@ DT_F16, DT_BF16, DT_F32, DT_I32 = 0, 1, 2, 3
 OK, ERR_BAD_PARAM, ERR_LDS_BUDGET, ERR_NO_INSTANCE, ERR_HIP, ERR_ALIGNMENT, ERR_NULL, ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6, -7
 OPT_SWIZZLE, OPT_SPIN_LIMIT, OPT_NUM_XCD, OPT_PRIO_MODE, OPT_PRODUCER_NAP, OPT_TILE_SYNC_BARRIER, OPT_STRAIGHT_LINE, OPT_SPLIT_K, OPT_BARRIER_EVERY_KSTEP = 0, 1, 2, 3, 4, 5, 6, 7, 8
 OPT_EVEN_ROUNDS = 9
+OPT_HALF_WIDTH = 11  # 256 x 128 tiles of the straight-line kernel: 0 never, 1 where the cost model prefers them (default), 2 always
 OPT_D_STORE_POLICY = 10  # 0: non-temporal stores of D where its rows lie on 128-byte lines (default), 1: always, 2: never
 
 if not os.path.exists(LIB_PATH):

@@ -20,8 +20,8 @@ CK_DECL_GEMM(launch_gemm_pc_bf16_m0) CK_DECL_GEMM(launch_gemm_pc_bf16_m1) CK_DEC
 #undef CK_DECL_GEMM
 hipError_t launch_gemm_pcb_f16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_pcb_bf16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
-hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep);
-hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep);
+hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, bool half_width);
+hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, bool half_width);
 bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves);
 constexpr int STREAM_K_MULTIPLE_HOST = 64;  // K extent of one loop body of the straight-line kernel
 hipError_t launch_gemm_fused_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
@@ -54,6 +54,7 @@ std::atomic<int> g_straight_line{1};
 std::atomic<int> g_even_rounds{1};
 std::atomic<int> g_split_k{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
 std::atomic<int> g_barrier_every_kstep{1};
+std::atomic<int> g_half_width{1};  // 256 x 128 tiles of the straight-line kernel: 0 never, 1 where the cost model prefers them, 2 always
 std::atomic<int> g_d_store_policy{0};  // 0: non-temporal stores of D where its rows lie on 128-byte lines, 1: always, 2: never
 constexpr int LINE_BYTES = 128;         // cache line of the vector memory path
 constexpr int SPLIT_K_MIN_SLICE = 1024;  // shortest K slice split-K will make (shorter ones lose more in the reduction pass than they gain)
@@ -229,29 +230,32 @@ int persistent_grid(int64_t tiles, int num_cus, int num_xcd, bool even_rounds) {
     return (int)(g < num_cus ? g : num_cus);
 }
 
-// Estimated duration (microseconds) of the straight-line kernel on `tiles` 256 x 256 tiles of an M x N product with K cut
-// into S slices, plus the reduction pass when S > 1. The constants are measurements of one MI355X on random operands:
-// a loop body (64 of K) takes 1.05 us while at most half of the 256 CUs multiply and the clock is free, and grows with
-// the number of active CUs once the device is power-limited (1.42 us with all of them); a work item costs about 3 us
-// of pipeline fill and drain; the items of a round store their 256 KiB each at the 4.6 TB/s the write path sustains;
-// the reduction pass reads S planes and writes D at 5.3 TB/s behind about 3 us of launch.
-double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus) {
+// Estimated duration (microseconds) of the straight-line kernel on `tiles` tiles (256 x 256, or 256 x 128 with
+// half_width) of an M x N product with K cut into S slices, plus the reduction pass when S > 1. The constants are
+// measurements of one MI355X on random operands: a loop body (64 of K) of a 256 x 256 tile takes 1.05 us while at most
+// half of the 256 CUs multiply and the clock is free, and grows with the number of active CUs once the device is
+// power-limited (1.42 us with all of them); a 256 x 128 tile's body has half the MFMAs and takes 0.585 of that time
+// at the power-limited clock but no less than 0.69 us (one barrier per 16 MFMAs); a work item costs about 3 us of pipeline fill and drain; the items of a round store their tile at the
+// 4.6 TB/s the write path sustains; the reduction pass reads S planes and writes D at 5.3 TB/s behind about 3 us of launch.
+constexpr double HALF_WIDTH_BODY = 0.585, HALF_WIDTH_BODY_MIN_US = 0.69;
+double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus, bool half_width) {
     const double items = (double)tiles * S;
     const double rounds = std::ceil(items / num_cus);
     const double active = items / rounds;   // workgroups (CUs) busy in a round
-    const double body_us = 1.05 * std::max(1.0, std::pow(active / 128.0, 0.43));
+    const double full_body_us = 1.05 * std::max(1.0, std::pow(active / 128.0, 0.43));
+    const double body_us = half_width ? std::max(HALF_WIDTH_BODY_MIN_US, HALF_WIDTH_BODY * full_body_us) : full_body_us;
     const double bodies = (double)K / S / ck::STREAM_K_MULTIPLE_HOST;
-    const double store_us = active * (256.0 * 1024.0) / 4.6e6;
+    const double store_us = active * (half_width ? 128.0 : 256.0) * 1024.0 / 4.6e6;
     double t = rounds * (bodies * body_us + store_us + 3.0);
     if (S > 1) t += 3.0 + (double)(S + 1) * (double)mn * 4.0 / 5.3e6;
     return t;
 }
 
-// Number of K slices the straight-line kernel uses for `tiles` 256 x 256 tiles (1: no split). policy 0: never;
+// Number of K slices the straight-line kernel uses for `tiles` tiles (1: no split). policy 0: never;
 // 1: automatic - with fewer tiles than CUs, the legal slice count whose estimated duration is shortest (a larger count
 // must win by 3 %: it costs scratch memory); >= 2: that many slices if legal, else the next smaller legal count.
 // Legal: slices of whole loop bodies and at least SPLIT_K_MIN_SLICE deep (any tile count, any N).
-int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, int policy) {
+int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, int policy, bool half_width) {
     if (policy == 0 || tiles <= 0) return 1;
     auto legal = [&](int c) { return K % (c * ck::STREAM_K_MULTIPLE_HOST) == 0 && K / c >= SPLIT_K_MIN_SLICE; };
     if (policy >= 2) {
@@ -261,13 +265,37 @@ int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, int policy) {
     }
     if (tiles >= num_cus) return 1;
     int best = 1;
-    double best_us = split_k_estimate_us(tiles, mn, K, 1, num_cus);
+    double best_us = split_k_estimate_us(tiles, mn, K, 1, num_cus, half_width);
     for (int c = 2; c <= 16; ++c) {
         if (!legal(c)) continue;
-        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus);
+        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus, half_width);
         if (us < 0.97 * best_us) { best = c; best_us = us; }
     }
     return best;
+}
+
+// How the straight-line kernel runs an M x N x K product on num_cus workgroups: tile width, K slices, and the
+// estimate that decided. 256 x 128 tiles where they are estimated at least 5 % faster (they fill a device that few
+// 256 x 256 tiles leave idle, at a lower rate per CU), or always / never by the option.
+struct StreamPlan {
+    bool half_width;
+    int slices;
+    int64_t tiles;
+    double us;
+};
+StreamPlan stream_plan(int M, int N, int K, int num_cus) {
+    const int64_t mn = (int64_t)M * N;
+    const int policy = g_split_k.load(), width = g_half_width.load();
+    auto plan = [&](bool half) {
+        const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + (half ? 127 : 255)) / (half ? 128 : 256));
+        const int slices = split_k_slices(tiles, mn, K, num_cus, policy, half);
+        return StreamPlan{half, slices, tiles, split_k_estimate_us(tiles, mn, K, slices, num_cus, half)};
+    };
+    const StreamPlan full = plan(false);
+    if (width == 0) return full;
+    const StreamPlan half = plan(true);
+    if (width == 2) return half;
+    return half.us < 0.95 * full.us ? half : full;
 }
 
 // The tuning tuple the straight-line kernel is written for (it also needs K in whole loop bodies of 64).
@@ -294,8 +322,7 @@ size_t scratch_need(int M, int N, int K, bool operands_aligned, const ck::GemmTu
         need += scratch_round(((size_t)M + (size_t)N) * k * 2);
     }
     if (straight_line_tuple(t)) {
-        const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-        const int slices = split_k_slices(tiles, (int64_t)M * N, k, t.num_cus, g_split_k.load());
+        const int slices = stream_plan(M, N, k, t.num_cus).slices;
         if (slices > 1) need += scratch_round((size_t)slices * M * N * sizeof(float));
     }
     return need;
@@ -383,10 +410,16 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     a.split_chunk = 32;
     if (g_straight_line.load() &&
         gemm_stream_applies(a, t.tile_dim, t.segment_dim_k, t.num_stages, t.num_producer_waves, t.num_consumer_waves)) {
-        // Few tiles and a deep K: cut K into slices so that every CU has an item, partial products into
-        // a stream-ordered workspace, one reduction pass.
+        // Tile width and K slices from the cost model: few tiles and a deep K are cut into slices so that every CU
+        // has an item (partial products into scratch memory, one reduction pass); tile counts that leave much of the
+        // device idle take 256 x 128 tiles.
         const bool bek = g_barrier_every_kstep.load() != 0;
-        int slices = split_k_slices(tiles, (int64_t)M * N, K, t.num_cus, g_split_k.load());
+        const StreamPlan plan = stream_plan(M, N, K, t.num_cus);
+        int slices = plan.slices;
+        const bool half = plan.half_width;
+        const int64_t tiles = plan.tiles;
+        if (half) a.tiles_n = (N + 127) / 128;
+        const int grid = persistent_grid(tiles, t.num_cus, a.num_xcd, g_even_rounds.load() != 0);
         const long long count = (long long)M * N;
         float* ws = nullptr;
         if (slices > 1) {
@@ -397,7 +430,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             if (trc != CK_OK) slices = 1;
         }
         if (slices == 1) {
-            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a, bek) : launch_gemm_stream_bf16(dim3(grid), s, a, bek);
+            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a, bek, half) : launch_gemm_stream_bf16(dim3(grid), s, a, bek, half);
         } else {
             GemmArgs p = a;
             p.split_k = slices;
@@ -408,7 +441,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             p.nt_store = store_policy == 1 || (store_policy == 0 && whole_lines(ws, (int64_t)N * 4) && count * 4 % LINE_BYTES == 0);
             const int64_t items = tiles * slices;
             const int pgrid = (int)(items < t.num_cus ? items : t.num_cus);
-            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p, bek) : launch_gemm_stream_bf16(dim3(pgrid), s, p, bek);
+            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p, bek, half) : launch_gemm_stream_bf16(dim3(pgrid), s, p, bek, half);
             if (e == hipSuccess) {
                 const unsigned blocks = (unsigned)((count + 255) / 256 < 65535 * 8 ? (count + 255) / 256 : 65535 * 8);
                 const bool vec4 = !out16 && count % 4 == 0 && ((uintptr_t)D | (uintptr_t)(beta != 0.f ? C : nullptr)) % 16 == 0;
@@ -593,11 +626,10 @@ int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out)
         if (t256 * 2 >= num_cus) pick = pc_256;
         else if (tiles(128) * 2 >= num_cus) pick = fused_128;
     } else {
-        // the shortest of three estimates: the straight-line kernel with the slice count the launcher would choose
-        // (split_k_estimate_us), and the general kernel on 128 and on 64 tiles - one workgroup per CU, measured per
+        // the shortest of three estimates: the straight-line kernel with the tile width and slice count the launcher
+        // would choose (stream_plan), and the general kernel on 128 and on 64 tiles - one workgroup per CU, measured per
         // 128 of K: 1.4 us for a 128 x 128 tile, 0.65 us for a 64 x 64 tile, about 4 us per round besides
-        const int slices = split_k_slices(t256, (int64_t)M * N, kp, num_cus, g_split_k.load());
-        const double straight_us = split_k_estimate_us(t256, (int64_t)M * N, kp, slices, num_cus);
+        const double straight_us = stream_plan(M, N, kp, num_cus).us;
         auto general_us = [&](int t, double seg_us) { return std::ceil((double)tiles(t) / num_cus) * ((double)K / 128.0 * seg_us + 4.0); };
         const double us_128 = general_us(128, 1.4), us_64 = general_us(64, 0.65);
         if (straight_us <= us_128 && straight_us <= us_64) pick = straight_line;
@@ -678,6 +710,7 @@ int ckopt_set_option(int key, int value) {
         case 8: return g_barrier_every_kstep.exchange(value != 0);
         case 9: return g_even_rounds.exchange(value != 0);
         case 10: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_d_store_policy.exchange(value);
+        case 11: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_half_width.exchange(value);
         default: return ck::CK_ERR_BAD_PARAM;
     }
 }

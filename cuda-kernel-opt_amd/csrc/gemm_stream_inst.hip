@@ -1,13 +1,14 @@
-// Launchers of the straight-line 256 x 256 kernel (one instance per element type).
+// Launchers of the straight-line kernel (one instance per element type, schedule, K-tail form and tile width).
 #include "gemm_stream_kernel.hip.h"
 
 namespace ck {
 
 static_assert(STREAM_K_MULTIPLE == 64, "the host's slice rule assumes loop bodies of 64");
 
-template <typename DT, bool ODD_ONLY, bool KTAIL>
+template <typename DT, bool ODD_ONLY, bool KTAIL, int WTC>
 static hipError_t stream_launch_one(dim3 grid, hipStream_t stream, const GemmArgs& a) {
-    auto kern = gemm_stream_kernel<DT, ODD_ONLY, KTAIL>;
+    auto kern = gemm_stream_kernel<DT, ODD_ONLY, KTAIL, WTC>;
+    constexpr int lds_bytes = stream_lds_bytes(2 * WTC * 16);
     static bool opted[64] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -17,22 +18,27 @@ static hipError_t stream_launch_one(dim3 grid, hipStream_t stream, const GemmArg
         if (e != hipSuccess) return e;
         opted[dev] = true;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(512), STREAM_LDS_BYTES, stream, a);
+    hipLaunchKernelGGL(kern, grid, dim3(512), lds_bytes, stream, a);
     return hipGetLastError();
 }
 
 // K in whole loop bodies: the plain instance; otherwise (K a multiple of 8) the one whose last body masks the end of K
+template <typename DT, bool ODD_ONLY, int WTC>
+static hipError_t stream_launch_k(dim3 grid, hipStream_t stream, const GemmArgs& a) {
+    return a.K % STREAM_K_MULTIPLE == 0 ? stream_launch_one<DT, ODD_ONLY, false, WTC>(grid, stream, a) : stream_launch_one<DT, ODD_ONLY, true, WTC>(grid, stream, a);
+}
 template <typename DT, bool ODD_ONLY>
-static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a) {
-    return a.K % STREAM_K_MULTIPLE == 0 ? stream_launch_one<DT, ODD_ONLY, false>(grid, stream, a) : stream_launch_one<DT, ODD_ONLY, true>(grid, stream, a);
+static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a, bool half_width) {
+    return half_width ? stream_launch_k<DT, ODD_ONLY, 4>(grid, stream, a) : stream_launch_k<DT, ODD_ONLY, 8>(grid, stream, a);
 }
 
-// barrier_every_kstep selects the schedule with a barrier in both k-steps of a loop body
-hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep) {
-    return barrier_every_kstep ? stream_launch<f16_tag, false>(grid, stream, a) : stream_launch<f16_tag, true>(grid, stream, a);
+// barrier_every_kstep selects the schedule with a barrier in both k-steps of a loop body; half_width the 256 x 128 tiles
+// (a.tiles_n then counts tiles of 128 columns)
+hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, bool half_width) {
+    return barrier_every_kstep ? stream_launch<f16_tag, false>(grid, stream, a, half_width) : stream_launch<f16_tag, true>(grid, stream, a, half_width);
 }
-hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep) {
-    return barrier_every_kstep ? stream_launch<bf16_tag, false>(grid, stream, a) : stream_launch<bf16_tag, true>(grid, stream, a);
+hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, bool half_width) {
+    return barrier_every_kstep ? stream_launch<bf16_tag, false>(grid, stream, a, half_width) : stream_launch<bf16_tag, true>(grid, stream, a, half_width);
 }
 
 // what the kernel assumes about a launch (the caller falls back to the general fused kernel otherwise)

@@ -47,20 +47,31 @@ constexpr int STREAM_TILE = 256;
 constexpr int STREAM_SEGK = 32;
 constexpr int STREAM_STAGES = 5;
 constexpr int STREAM_K_MULTIPLE = 2 * STREAM_SEGK;  // one loop body
-constexpr int STREAM_LDS_BYTES = STREAM_STAGES * 2 * STREAM_TILE * STREAM_SEGK * 2;
+constexpr int STREAM_TILE_N_HALF = 128;   // the half-width form: 256 x 128 tiles (wave tiles of 64 x 64)
+// bytes of the ring for tiles of 256 x tile_n
+constexpr int stream_lds_bytes(int tile_n) { return STREAM_STAGES * (STREAM_TILE + tile_n) * STREAM_SEGK * 2; }
+constexpr int STREAM_LDS_BYTES = stream_lds_bytes(STREAM_TILE);
 
 // KTAIL: K is a multiple of 8 but not of 64. The last loop body of a tile then reaches past K: its loads take
 // per-lane offsets in which every 16-byte chunk at or beyond K lies outside the descriptor (reads as zeros), chosen
 // by a scalar branch inside the load's asm statement, so that nothing is added to the other bodies but two scalar
 // instructions per load. Launches with K % 64 == 0 run the instance without any of it.
-template <typename DT, bool ODD_ONLY, bool KTAIL>
+// WTC: 16-column blocks per wave tile. 8: 256 x 256 tiles (wave tiles of 64 x 128); 4: 256 x 128 tiles (wave tiles of
+// 64 x 64) for launches whose 256 x 256 tiles would leave most of the device idle - twice the tiles, half the MFMAs
+// per k-step and wave, a ring of 24 KiB quarters, one load pair of Bt per wave and body instead of two.
+template <typename DT, bool ODD_ONLY, bool KTAIL, int WTC>
 __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     constexpr int TILE = STREAM_TILE, NQ = STREAM_STAGES;
-    constexpr int WTR = 4, WTC = 8;          // 16 x 16 blocks per wave tile (64 x 128)
+    constexpr int WTR = 4;                   // 16 x 16 blocks per wave tile: WTR x WTC (64 rows x 128 or 64 columns)
+    constexpr int TILE_N = 2 * WTC * 16;     // two wave tiles side by side
     constexpr int RB = STREAM_SEGK * 2;      // bytes per LDS row
-    constexpr int OPB = TILE * RB;           // one operand's part of a quarter
-    constexpr int QB = 2 * OPB;              // one quarter
-    constexpr int LPB = 8;                   // loads per wave and body: (A, Bt) x (rows w, w + 8) x (two halves)
+    constexpr int OPB = TILE * RB;           // A's part of a quarter
+    constexpr int OPB_B = TILE_N * RB;       // Bt's part
+    constexpr int QB = OPB + OPB_B;          // one quarter
+    constexpr int B_PAIRS = TILE_N / 128;    // load pairs of Bt per wave and body (16 rows each)
+    constexpr int LPB = (2 + B_PAIRS) * 2;   // loads per wave and body: (A rows w, w + 8; Bt rows w [, w + 8]) x (two halves)
+    constexpr int EVEN_LOADS = 4;            // of those, issued in the even k-step when every k-step has a barrier: A's
+    static_assert(WTC == 8 || WTC == 4, "wave tiles of 64 x 128 or 64 x 64");
     // Stores one wave issues in the epilogue of an interior tile. The landing wait of the body behind an epilogue
     // counts them (they sit between the loads in flight and the new ones), so the loops below and the wait
     // immediates are written in terms of the same constants.
@@ -71,11 +82,12 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     static_assert(WTC % F32_GROUP == 0 && WTC % H16_GROUP == 0, "whole groups per wave-tile row");
     static_assert(EPILOGUE_STORES_16 * 2 == EPILOGUE_STORES, "count_stores selects between the two with a shift by one");
     constexpr int PRE = 1;               // columns of MFMAs in front of the barrier
-    constexpr int LOAD_COL_0 = 3;  // columns behind which a k-step's two load pairs are issued
-    constexpr int LOAD_COL_1 = 6;
-    static_assert(PRE >= 1 && (WTC - PRE) * 2 >= WTR + WTC && LOAD_COL_0 >= PRE && LOAD_COL_1 > LOAD_COL_0 && LOAD_COL_1 < WTC, "schedule");
+    constexpr int LOAD_COL_0 = WTC == 8 ? 3 : 1;  // columns behind which a k-step's two load pairs are issued
+    constexpr int LOAD_COL_1 = WTC == 8 ? 6 : 3;
+    constexpr int FPC = (WTR + WTC + (WTC - PRE) - 1) / (WTC - PRE);   // fragments of the next k-step fetched per column
+    static_assert(PRE >= 1 && (WTC - PRE) * FPC >= WTR + WTC && LOAD_COL_0 >= PRE && LOAD_COL_1 > LOAD_COL_0 && LOAD_COL_1 < WTC, "schedule");
     static_assert(LPB + EPILOGUE_STORES < 64 && EPILOGUE_STORES_16 < EPILOGUE_STORES, "the wait immediates must fit the 6-bit counter");
-    static_assert(STREAM_LDS_BYTES <= LDS_BYTES_PER_CU, "the ring is all of the LDS");
+    static_assert(NQ * QB == stream_lds_bytes(TILE_N) && NQ * QB <= LDS_BYTES_PER_CU, "the ring (all of the LDS for 256 x 256 tiles)");
 
     extern __shared__ __attribute__((aligned(1024))) char ck_smem[];
     const uint32_t ring_base = (uint32_t)(uintptr_t)(CK_LDS char*)ck_smem;
@@ -138,8 +150,8 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             int slice = 0;
             const int64_t tc = item_tile(slot + (int64_t)l_tile * grid, slice);
             const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
-            const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE);
-            const int ra = g.M - row_a < TILE ? g.M - row_a : TILE, rb = g.N - row_b < TILE ? g.N - row_b : TILE;
+            const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE_N);
+            const int ra = g.M - row_a < TILE ? g.M - row_a : TILE, rb = g.N - row_b < TILE_N ? g.N - row_b : TILE_N;
             const int64_t k0 = (int64_t)slice * kslice_bytes;  // the slice starts k0 bytes into every row
             // (the descriptor's extent is counted from the shifted base: the last row ends k0 bytes early)
             rsrc_a = make_rsrc((const char*)g.A + (int64_t)row_a * pitch32 + k0, (uint32_t)ra * pitch32 - (uint32_t)k0);
@@ -159,12 +171,13 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         if constexpr (KTAIL)   // (kept in one opaque scalar register, like stores_in_flight below)
             asm volatile("s_mov_b32 %0, %1" : "=s"(l_tail) : "s"(__builtin_amdgcn_readfirstlane((uint32_t)(l_koff + STREAM_K_MULTIPLE * 2 > kslice_bytes))));
     };
-    // Load pair P (0, 1: A rows 16w.. / 16(w+8)..; 2, 3: Bt likewise) of the body at l_koff: the two
+    // Load pair P (0, 1: A rows 16w.. / 16(w+8)..; 2, 3: Bt likewise; 256 x 128 tiles have no pair 3) of the body at l_koff: the two
     // halves of each row's line, back to back, into the quarters at byte offsets q_lo and q_hi.
     auto issue_pair = [&](auto index, uint32_t q_lo, uint32_t q_hi) __attribute__((always_inline)) {
         constexpr int P = decltype(index)::value;
         constexpr bool IS_A = P < 2;
         constexpr int HI = P % 2;
+        if constexpr (P == 3 && B_PAIRS < 2) return;
         const uint32_t dst = dst_w + (uint32_t)((IS_A ? 0 : OPB) + HI * 8 * 1024);
         if constexpr (KTAIL) {
             dma_load_b128_select(IS_A ? rsrc_a : rsrc_b, dst + q_lo, HI ? loff_hi : loff_lo, HI ? toff_hi[0] : toff_lo[0], l_koff, l_tail);
@@ -223,8 +236,8 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             asm volatile("s_cmp_lg_u32 %0, 0\n\ts_cbranch_scc1 1f\n\ts_waitcnt vmcnt(%1)\n1:\n\t"
                          "s_cmp_eq_u32 %0, 2\n\ts_cbranch_scc1 2f\n\ts_waitcnt vmcnt(%2)\n2:\n\ts_waitcnt vmcnt(%3)"
                          :
-                         : "s"(stores_in_flight), "n"(ODD_ONLY ? 0 : LPB / 2), "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES_16),
-                           "n"((ODD_ONLY ? 0 : LPB / 2) + EPILOGUE_STORES)
+                         : "s"(stores_in_flight), "n"(ODD_ONLY ? 0 : EVEN_LOADS), "n"((ODD_ONLY ? 0 : EVEN_LOADS) + EPILOGUE_STORES_16),
+                           "n"((ODD_ONLY ? 0 : EVEN_LOADS) + EPILOGUE_STORES)
                          : "memory", "scc");
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -239,8 +252,8 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
         for (int j = PRE; j < WTC; ++j) {
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const int f = (j - PRE) * 2 + q;
+            for (int q = 0; q < FPC; ++q) {
+                const int f = (j - PRE) * FPC + q;
                 if (f < WTR) fa[1 - P][f] = *(const CK_LDS u32x4*)(uintptr_t)(pa + (uint32_t)(f * 16 * RB));
                 else if (f < WTR + WTC) fb[1 - P][f - WTR] = *(const CK_LDS u32x4*)(uintptr_t)(pb + (uint32_t)((f - WTR) * 16 * RB));
             }
@@ -250,11 +263,16 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             // A in the even k-step, those of Bt in the odd one
             if constexpr (ODD_ONLY) {
                 // all four pairs in the odd k-step, behind its barrier (the only one of the body)
-                if constexpr (P == 1) {
+                if constexpr (P == 1 && WTC == 8) {
                     if (j == 2) issue_pair(std::integral_constant<int, 0>{}, q4, q0);
                     if (j == 4) issue_pair(std::integral_constant<int, 1>{}, q4, q0);
                     if (j == 6) issue_pair(std::integral_constant<int, 2>{}, q4, q0);
                     if (j == 7) issue_pair(std::integral_constant<int, 3>{}, q4, q0);
+                }
+                if constexpr (P == 1 && WTC == 4) {
+                    if (j == 1) issue_pair(std::integral_constant<int, 0>{}, q4, q0);
+                    if (j == 2) issue_pair(std::integral_constant<int, 1>{}, q4, q0);
+                    if (j == 3) issue_pair(std::integral_constant<int, 2>{}, q4, q0);
                 }
             } else {
                 if (j == LOAD_COL_0) issue_pair(std::integral_constant<int, 2 * P>{}, q4, q0);
@@ -317,11 +335,11 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             GemmArgs go = g;  // a K slice writes its own plane of the workspace D points at
             go.D = g.D + (size_t)slice * ((size_t)g.M * g.N);
             const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
-            const int n_base = rc.col * TILE + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
+            const int n_base = rc.col * TILE_N + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
             // vec_cols: every column of the tile is inside the matrix, one vector access per block (rows past M are
             // skipped lane by lane); interior: every row as well, so every wave issues exactly the stores that the next
             // body's landing wait counts
-            const bool vec_cols = g.vec_store && (rc.col + 1) * TILE <= g.N;
+            const bool vec_cols = g.vec_store && (rc.col + 1) * TILE_N <= g.N;
             const bool interior = vec_cols && (rc.row + 1) * TILE <= g.M;
             // rows of D on 128-byte lines: the stores below fill whole lines and bypass L2 retention; otherwise every
             // 128-byte run of a row straddles two lines, and ordinary stores let the halves meet in L2 (N = 4097,
@@ -337,7 +355,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                 const int src0 = ((lane >> 3) + 16 * (piece & 3)) * 4;  // byte address of the source lane, t = 0
                 const bool second = piece >= 4;
                 const int64_t row0 = (int64_t)(rc.row * TILE + R * WTR * 16 + (lane >> 3));
-                const int col0 = rc.col * TILE + Cc * WTC * 16 + piece * 4;
+                const int col0 = rc.col * TILE_N + Cc * WTC * 16 + piece * 4;
                 const float alpha = g.alpha, beta = g.beta;
 #pragma unroll
                 for (int i = 0; i < WTR; ++i) {
@@ -375,7 +393,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                 const bool low_rows = lr < 8;
                 const int unit = ((lg & 1) * 2 + (lg >> 1)) * 8;   // column of the lane's piece inside a pair's 32
                 const int64_t row0 = (int64_t)(rc.row * TILE + R * WTR * 16 + (lr & 7));
-                const int col0 = rc.col * TILE + Cc * WTC * 16 + unit;
+                const int col0 = rc.col * TILE_N + Cc * WTC * 16 + unit;
                 const float alpha = g.alpha;
                 typedef uint32_t pair_u32 __attribute__((ext_vector_type(2)));
                 auto packed_pair = [&](f32x4 x0, f32x4 x1) __attribute__((always_inline)) {

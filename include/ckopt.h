@@ -206,6 +206,10 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  *        start anywhere make every 128-byte run of a row straddle two lines, and only ordinary stores let the parts
  *        meet in L2 before they reach memory (bf16 6143 x 4097 x 3072: 138 us against 164). 1: always non-temporal;
  *        2: never.
+ * key 11: tile width of the straight-line kernel. 1 (default): 256 x 128 tiles (wave tiles of 64 x 64, twice the tiles,
+ *        0.86 of the rate on a full device) where the launcher's cost model gives them at least 5 % less time than
+ *        256 x 256 tiles - tile counts that leave much of the device idle (2560^3: 100 tiles, 53 us -> 37 us);
+ *        0: never; 2: always. tile_dim stays 256 in the launcher's parameters.
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

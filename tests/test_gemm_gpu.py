@@ -565,10 +565,14 @@ def test_straight_line_kernel_any_k(ck, M, N, K):
         bt = ck.fill_int(dt, (N, K), 98, 1, -2, 2)
         c = ck.fill_int(ck.DT_F32, (M, N), 98, 2, -3, 3)
         exact = G.as_f64(dt == ck.DT_BF16, a) @ G.as_f64(dt == ck.DT_BF16, bt).T
-        for cus in (256, 3):
+        for cus, width in ((256, 0), (3, 0), (256, 2), (3, 2)):   # 256 x 256 tiles and 256 x 128 tiles
             t = _straight_line_tuning(ck, cus)
-            assert np.array_equal(G.run_gemm(ck, dt, a, bt, t=t), exact.astype(np.float32)), (M, N, K, dt, cus)
-            assert np.array_equal(G.run_gemm(ck, dt, a, bt, c, -1.0, 2.0, t=t), (2.0 * c - exact).astype(np.float32))
+            prev = ck.set_option(ck.OPT_HALF_WIDTH, width)
+            try:
+                assert np.array_equal(G.run_gemm(ck, dt, a, bt, t=t), exact.astype(np.float32)), (M, N, K, dt, cus, width)
+                assert np.array_equal(G.run_gemm(ck, dt, a, bt, c, -1.0, 2.0, t=t), (2.0 * c - exact).astype(np.float32)), (width,)
+            finally:
+                ck.set_option(ck.OPT_HALF_WIDTH, prev)
     order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b",
                             "tile_group_m", "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
     if K % 8:
@@ -769,17 +773,64 @@ def test_split_k_bit_exact(ck, M, N, K, slices, cus, dt_name):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("M,N,K", [(512, 512, 256), (700, 390, 1024), (1024, 768, 4096), (260, 1000, 200)])
+def test_half_width_tiles_exact(ck, M, N, K):
+    """256 x 128 tiles of the straight-line kernel, forced: fp32 and 16-bit C / D (whole-line and element-wise epilogues),
+    with and without C, K slices, few and many workgroups; exact on small integers, every element written."""
+    prev = ck.set_option(ck.OPT_HALF_WIDTH, 2)
+    try:
+        for dt in (ck.DT_F16, ck.DT_BF16):
+            is_bf = dt == ck.DT_BF16
+            tdt = torch.bfloat16 if is_bf else torch.float16
+            a = ck.fill_int(dt, (M, K), 61, 0, -1, 1)
+            bt = ck.fill_int(dt, (N, K), 61, 1, -1, 1)
+            c = ck.fill_int(ck.DT_F32, (M, N), 61, 2, -3, 3)
+            exact = G.as_f64(is_bf, a) @ G.as_f64(is_bf, bt).T
+            for cus in (256, 6):
+                t = _straight_line_tuning(ck, cus)
+                for split in (0, 1, 2):
+                    before = ck.set_option(ck.OPT_SPLIT_K, split)
+                    try:
+                        assert np.array_equal(G.run_gemm(ck, dt, a, bt, t=t), exact.astype(np.float32)), (dt, cus, split)
+                        assert np.array_equal(G.run_gemm(ck, dt, a, bt, c, 0.5, -2.0, t=t), (0.5 * exact - 2.0 * c).astype(np.float32)), (dt, cus, split)
+                        da, db = G.to_dev(a), G.to_dev(bt)
+                        dd = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+                        ck.gemm_shmem_tc_async_opt_port_lp(dt, da, db, None, dd, 0.0625, 0.0, M, N, K, t["tile_dim"], t["segment_dim_k"],
+                                                           t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                                           t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                                           t["num_consumer_warps"], t["num_sms"])
+                        assert ck.device_status() == 0
+                        want16 = torch.from_numpy((exact * 0.0625).astype(np.float32)).to(tdt).float().numpy()
+                        assert np.array_equal(dd.float().cpu().numpy(), want16), (dt, cus, split)
+                    finally:
+                        ck.set_option(ck.OPT_SPLIT_K, before)
+    finally:
+        ck.set_option(ck.OPT_HALF_WIDTH, prev)
+
+
+def test_half_width_tiles_chosen_for_100_tiles_full_size(ck, oracle):
+    # 2560^3: 100 tiles of 256 x 256 on 256 CUs; the launcher takes 256 x 128 tiles by itself. Whole matrix against the oracle.
+    M = N = K = 2560
+    full_size_check(ck, oracle, ck.DT_F16, oracle.DT_F16, M, N, K, (_straight_line_tuning(ck),), lambda s, shape: ck.fill_uniform(ck.DT_F16, shape, 0xC0FFEE09, s))
+
+
 def test_automatic_split_k_of_128_tiles_exact(ck):
-    # 128 tiles on 256 CUs with a deep K: the automatic rule cuts K in two (256 work items); exact on small integers
+    # 128 tiles on 256 CUs with a deep K: with 256 x 256 tiles only, the automatic rule cuts K in two (256 work items);
+    # with both widths it takes 256 tiles of 256 x 128 and no slices. Exact on small integers either way.
     M, N, K = 2048, 4096, 8192
     t = _straight_line_tuning(ck)
     order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b",
                             "tile_group_m", "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
-    assert ck.gemm_workspace_bytes(M, N, K, True, *order) == 2 * M * N * 4 + 256
     a = ck.fill_int(ck.DT_F16, (M, K), 97, 0, -1, 1)
     bt = ck.fill_int(ck.DT_F16, (N, K), 97, 1, -1, 1)
     want = (a.astype(np.float32) @ bt.astype(np.float32).T)   # sums of at most 8192 terms of -1, 0, 1: exact in fp32
-    assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want)
+    for width, planes in ((0, 2), (1, 0)):
+        prev = ck.set_option(ck.OPT_HALF_WIDTH, width)
+        try:
+            assert ck.gemm_workspace_bytes(M, N, K, True, *order) == (planes * M * N * 4 + 256 if planes else 0)
+            assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want), width
+        finally:
+            ck.set_option(ck.OPT_HALF_WIDTH, prev)
 
 
 def test_split_k_against_the_oracle_and_the_single_pass(ck, oracle):
@@ -1030,7 +1081,8 @@ def test_random_tunings_entry_points_and_options_exact(ck):
         dt = ck.DT_F16 if rng.random() < 0.5 else ck.DT_BF16
         alpha, beta = float(rng.choice([1.0, 2.0, -0.5])), float(rng.choice([0.0, 0.0, -1.0, 2.0]))
         opts = {ck.OPT_SPLIT_K: int(rng.choice([0, 1, 1, 2, 3, 4, 8])), ck.OPT_BARRIER_EVERY_KSTEP: int(rng.integers(0, 2)),
-                ck.OPT_EVEN_ROUNDS: int(rng.integers(0, 2)), ck.OPT_TILE_SYNC_BARRIER: int(rng.integers(0, 2))}
+                ck.OPT_EVEN_ROUNDS: int(rng.integers(0, 2)), ck.OPT_TILE_SYNC_BARRIER: int(rng.integers(0, 2)),
+                ck.OPT_HALF_WIDTH: int(rng.integers(0, 3)), ck.OPT_D_STORE_POLICY: int(rng.integers(0, 3))}
         entry = int(rng.integers(0, 3))
         if ck.check_gemm_tuning(*order) != ck.OK:
             continue

@@ -381,15 +381,17 @@ class StreamModel:
     STORES = 32
 
     def __init__(self, waves, bodies_per_item, items, rng, imm=4, imm_stores=36, count_stores=True, completion_rate=0.35, slow_wave=None,
-                 odd_only=False):
+                 odd_only=False, bt_pairs=2, stores=32):
         self.n, self.nb, self.items, self.rng = waves, bodies_per_item, items, rng
         self.completion_rate = completion_rate                       # how eagerly the memory system answers
         self.slow_wave = slow_wave                                   # a wave whose operations complete 50 times more rarely
         self.odd_only = odd_only                                     # no barrier and no loads in the even k-step (immediates 0 / 32)
         self.imm, self.imm_stores, self.count_stores = imm, imm_stores, count_stores
+        self.bt_pairs, self.stores = bt_pairs, stores                # 256 x 128 tiles: one load pair of Bt per wave and body, 16 stores per epilogue
+        self.slots = 2 + bt_pairs
         self.total = 2 * bodies_per_item * items                     # k-steps in the stream
         # per quarter and wave, per load of a k-step (A rows 16w.., A rows 16(w+8).., Bt likewise): k-step it holds
-        self.holds = [[[-1, -1, -1, -1] for _ in range(waves)] for _ in range(5)]
+        self.holds = [[[-1] * self.slots for _ in range(waves)] for _ in range(5)]
         self.queue = [[] for _ in range(waves)]                       # per wave: FIFO of ops
         self.arrived, self.generation = 0, 0
         self.errors = []
@@ -406,13 +408,13 @@ class StreamModel:
 
     def read(self, quarter, kstep):
         for w in range(self.n):
-            if self.holds[quarter][w] != [kstep] * 4:
+            if self.holds[quarter][w] != [kstep] * self.slots:
                 self.errors.append("k-step %d read from quarter %d: wave %d's share holds %s" % (kstep, quarter, w, self.holds[quarter][w]))
 
     def issue_pairs(self, w, operand, even_kstep, body_kstep):
         # two pairs = four loads of the body whose even k-step is body_kstep, issued in (or before) the body
         # of even k-step even_kstep, which fixes the quarters: lo halves -> body_kstep % 5, hi halves -> + 1
-        for pair in range(2):
+        for pair in range(2 if operand == 0 else self.bt_pairs):
             for half in range(2):
                 k = body_kstep + half
                 self.queue[w].append(("load", k % 5, 2 * operand + pair, k if k < self.total else -2))
@@ -433,7 +435,7 @@ class StreamModel:
         for body in (0, 1):
             for operand in (0, 1):
                 self.issue_pairs(w, operand, 0, 2 * body)
-        yield from wait(8)
+        yield from wait(2 * self.slots)
         yield from barrier()
         self.read(0, 0)
         stores_in_flight = False
@@ -457,7 +459,7 @@ class StreamModel:
             self.issue_pairs(w, 1, j, j + 4)
             stores_in_flight = False
             if (j + 2) % (2 * self.nb) == 0:                          # the item ends: epilogue
-                for _ in range(self.STORES):
+                for _ in range(self.stores):
                     self.queue[w].append(("store",))
                 stores_in_flight = self.count_stores
             yield
@@ -482,7 +484,10 @@ class StreamModel:
 
 
 # the two schedules of the kernel: a barrier in every k-step (immediates 4 / 36), or in the odd k-step only (0 / 32)
-SCHEDULES = {"barrier_every_kstep": dict(imm=4, imm_stores=36, odd_only=False), "odd_only": dict(imm=0, imm_stores=32, odd_only=True)}
+SCHEDULES = {"barrier_every_kstep": dict(imm=4, imm_stores=36, odd_only=False), "odd_only": dict(imm=0, imm_stores=32, odd_only=True),
+             # 256 x 128 tiles: six loads per body (A's four in the even k-step as before, Bt's two in the odd one), 16 stores per epilogue
+             "half_width_barrier_every_kstep": dict(imm=4, imm_stores=20, odd_only=False, bt_pairs=1, stores=16),
+             "half_width_odd_only": dict(imm=0, imm_stores=16, odd_only=True, bt_pairs=1, stores=16)}
 
 
 @pytest.mark.parametrize("schedule", sorted(SCHEDULES))
@@ -516,6 +521,14 @@ def test_stream_model_detects_wrong_immediates():
         caught = 0
         for seed in range(20):
             m = StreamModel(8, 2, 4, random.Random(seed), imm=imm, imm_stores=imm_stores, completion_rate=0.3, slow_wave=seed % 8, odd_only=True)
+            m.run()
+            caught += bool(m.errors)
+        assert caught > 0
+    # 256 x 128 tiles (16 stores per epilogue): one store too many allowed in flight, and the full-width immediate
+    for imm_stores in (21, 36):
+        caught = 0
+        for seed in range(20):
+            m = StreamModel(8, 1, 6, random.Random(seed), imm=4, imm_stores=imm_stores, completion_rate=0.3, slow_wave=seed % 8, bt_pairs=1, stores=16)
             m.run()
             caught += bool(m.errors)
         assert caught > 0
