@@ -357,31 +357,57 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                 const int64_t row0 = (int64_t)(rc.row * TILE + R * WTR * 16 + (lane >> 3));
                 const int col0 = rc.col * TILE_N + Cc * WTC * 16 + piece * 4;
                 const float alpha = g.alpha, beta = g.beta;
+                // store s of the epilogue: block row i, group of two block columns j, half tt
+                constexpr int GROUPS = WTC / F32_GROUP;
+                auto exchanged = [&](int i, int j, int tt) __attribute__((always_inline)) {
+                    f32x4 v;
 #pragma unroll
-                for (int i = 0; i < WTR; ++i) {
+                    for (int e = 0; e < 4; ++e) {
+                        const float x0 = acc[i][j][e], x1 = acc[i][j + 1][e];
+                        const int a0 = __builtin_amdgcn_ds_bpermute(src0 + tt * 32, __float_as_int(x0));
+                        const int a1 = __builtin_amdgcn_ds_bpermute(src0 + tt * 32, __float_as_int(x1));
+                        v[e] = __int_as_float(second ? a1 : a0) * alpha;
+                    }
+                    return v;
+                };
+                auto put = [&](int64_t off, f32x4 v) __attribute__((always_inline)) {
+                    if (nt_store) store_b128_nt(go.D + off, __builtin_bit_cast(u32x4, v));
+                    else *(f32x4_u*)(go.D + off) = v;
+                };
+                if (beta == 0.f) {
 #pragma unroll
-                    for (int j = 0; j < WTC; j += F32_GROUP) {
+                    for (int i = 0; i < WTR; ++i) {
 #pragma unroll
-                        for (int tt = 0; tt < STORES_PER_GROUP; ++tt) {
-                            f32x4 v;
+                        for (int j = 0; j < WTC; j += F32_GROUP) {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                const float x0 = acc[i][j][e], x1 = acc[i][j + 1][e];
-                                const int a0 = __builtin_amdgcn_ds_bpermute(src0 + tt * 32, __float_as_int(x0));
-                                const int a1 = __builtin_amdgcn_ds_bpermute(src0 + tt * 32, __float_as_int(x1));
-                                v[e] = __int_as_float(second ? a1 : a0) * alpha;
-                            }
-                            const int64_t row = row0 + i * 16 + tt * 8;
-                            const int64_t off = row * g.N + (col0 + j * 16);
-                            if (row < g.M) {
-                                if (beta != 0.f) v += *(const f32x4_u*)(go.C + off) * beta;
-                                if (nt_store) store_b128_nt(go.D + off, __builtin_bit_cast(u32x4, v));
-                                else *(f32x4_u*)(go.D + off) = v;
+                            for (int tt = 0; tt < STORES_PER_GROUP; ++tt) {
+                                const f32x4 v = exchanged(i, j, tt);
+                                const int64_t row = row0 + i * 16 + tt * 8;
+                                if (row < g.M) put(row * g.N + (col0 + j * 16), v);
                             }
                         }
                     }
+                } else {
+                    // C is read C_DEPTH stores ahead of its use: the loads of a wave would otherwise wait for memory one
+                    // by one between the stores (a load may not pass the store in front of it)
+                    constexpr int C_DEPTH = 4;
+                    f32x4 cv[C_DEPTH];
+                    auto row_of = [&](int st) { return row0 + (st / (GROUPS * STORES_PER_GROUP)) * 16 + (st % STORES_PER_GROUP) * 8; };
+                    auto off_of = [&](int st) { return row_of(st) * g.N + (col0 + ((st / STORES_PER_GROUP) % GROUPS) * F32_GROUP * 16); };
+                    auto fetch = [&](int st) __attribute__((always_inline)) {
+                        return row_of(st) < g.M ? (f32x4)*(const f32x4_u*)(go.C + off_of(st)) : f32x4{0.f, 0.f, 0.f, 0.f};
+                    };
+#pragma unroll
+                    for (int st = 0; st < C_DEPTH; ++st) cv[st] = fetch(st);
+#pragma unroll
+                    for (int st = 0; st < EPILOGUE_STORES; ++st) {
+                        f32x4 v = exchanged(st / (GROUPS * STORES_PER_GROUP), ((st / STORES_PER_GROUP) % GROUPS) * F32_GROUP, st % STORES_PER_GROUP);
+                        v += cv[st % C_DEPTH] * beta;
+                        if (row_of(st) < g.M) put(off_of(st), v);
+                        if (st + C_DEPTH < EPILOGUE_STORES) cv[st % C_DEPTH] = fetch(st + C_DEPTH);
+                    }
                 }
-            } else if (interior && g.out16 && d16_misaligned == 0 && g.beta == 0.f) {
+            } else if (interior && g.out16 && d16_misaligned == 0) {
                 // 16-bit output in whole 128-byte lines, 16 bytes per lane. A lane's 4 results of a block are
                 // 8 bytes, so two neighbouring blocks swap their odd and even 16-lane rows
                 // (v_permlane16_swap): lane group G = lane / 16 then holds the 8 columns 8 (G / 2) .. of block
@@ -394,10 +420,29 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                 const int unit = ((lg & 1) * 2 + (lg >> 1)) * 8;   // column of the lane's piece inside a pair's 32
                 const int64_t row0 = (int64_t)(rc.row * TILE + R * WTR * 16 + (lr & 7));
                 const int col0 = rc.col * TILE_N + Cc * WTC * 16 + unit;
-                const float alpha = g.alpha;
+                const float alpha = g.alpha, beta = g.beta;
+                // C (beta not zero) is read in the accumulators' own layout, 8 bytes per lane and block (columns 4 lg ..
+                // of row lr), one group of four blocks ahead of its use, and added in fp32 before the one rounding
+                const bool with_c = beta != 0.f;
+                const unsigned short* c16 = (const unsigned short*)go.C;
+                const int64_t c_lane = (int64_t)(rc.row * TILE + R * WTR * 16 + lr) * g.N + (rc.col * TILE_N + Cc * WTC * 16 + lg * 4);
                 typedef uint32_t pair_u32 __attribute__((ext_vector_type(2)));
-                auto packed_pair = [&](f32x4 x0, f32x4 x1) __attribute__((always_inline)) {
-                    const f32x4 v0 = x0 * alpha, v1 = x1 * alpha;
+                auto fetch_c = [&](int i, int j, pair_u32 (&c)[H16_GROUP]) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int b = 0; b < H16_GROUP; ++b)
+                        c[b] = with_c ? *(const pair_u32*)(c16 + c_lane + (int64_t)(i * 16) * g.N + (j + b) * 16) : pair_u32{0u, 0u};
+                };
+                auto scaled = [&](f32x4 x, pair_u32 c) __attribute__((always_inline)) {
+                    f32x4 v = x * alpha;
+                    if (with_c) {
+                        v[0] += Out16<DT>::load((unsigned short)(c[0] & 0xffffu)) * beta;
+                        v[1] += Out16<DT>::load((unsigned short)(c[0] >> 16)) * beta;
+                        v[2] += Out16<DT>::load((unsigned short)(c[1] & 0xffffu)) * beta;
+                        v[3] += Out16<DT>::load((unsigned short)(c[1] >> 16)) * beta;
+                    }
+                    return v;
+                };
+                auto packed_pair = [&](f32x4 v0, f32x4 v1) __attribute__((always_inline)) {
                     const uint32_t p00 = (uint32_t)Out16<DT>::store(v0[0]) | ((uint32_t)Out16<DT>::store(v0[1]) << 16);
                     const uint32_t p01 = (uint32_t)Out16<DT>::store(v0[2]) | ((uint32_t)Out16<DT>::store(v0[3]) << 16);
                     const uint32_t p10 = (uint32_t)Out16<DT>::store(v1[0]) | ((uint32_t)Out16<DT>::store(v1[1]) << 16);
@@ -406,12 +451,17 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                     const pair_u32 s1 = __builtin_amdgcn_permlane16_swap(p01, p11, false, false);
                     return u32x4{s0[0], s1[0], s0[1], s1[1]};
                 };
+                constexpr int GROUPS16 = WTC / H16_GROUP;
+                pair_u32 cq[2][H16_GROUP];
+                fetch_c(0, 0, cq[0]);
 #pragma unroll
                 for (int i = 0; i < WTR; ++i) {
 #pragma unroll
                     for (int j = 0; j < WTC; j += H16_GROUP) {
-                        const u32x4 first = packed_pair(acc[i][j], acc[i][j + 1]);
-                        const u32x4 second = packed_pair(acc[i][j + 2], acc[i][j + 3]);
+                        const int gi = i * GROUPS16 + j / H16_GROUP;   // this group; the next one's C goes into the other buffer
+                        if (gi + 1 < WTR * GROUPS16) fetch_c((gi + 1) / GROUPS16, ((gi + 1) % GROUPS16) * H16_GROUP, cq[(gi + 1) % 2]);
+                        const u32x4 first = packed_pair(scaled(acc[i][j], cq[gi % 2][0]), scaled(acc[i][j + 1], cq[gi % 2][1]));
+                        const u32x4 second = packed_pair(scaled(acc[i][j + 2], cq[gi % 2][2]), scaled(acc[i][j + 3], cq[gi % 2][3]));
                         u32x4 other;  // the second pair's piece of the row 8 away
 #pragma unroll
                         for (int e = 0; e < 4; ++e)

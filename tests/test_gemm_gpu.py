@@ -808,6 +808,35 @@ def test_half_width_tiles_exact(ck, M, N, K):
         ck.set_option(ck.OPT_HALF_WIDTH, prev)
 
 
+@pytest.mark.parametrize("M,N,K", [(512, 512, 128), (700, 520, 128), (256, 1024, 192)])
+def test_straight_line_16_bit_output_with_c(ck, M, N, K):
+    """16-bit C and D with beta != 0 on the straight-line kernel: interior tiles read C in the accumulators' layout and
+    store whole lines, edge tiles go element by element; both tile widths; exact (every value is a small integer)."""
+    for dt in (ck.DT_F16, ck.DT_BF16):
+        is_bf = dt == ck.DT_BF16
+        tdt = torch.bfloat16 if is_bf else torch.float16
+        a = ck.fill_int(dt, (M, K), 63, 0, -1, 1)
+        bt = ck.fill_int(dt, (N, K), 63, 1, -1, 1)
+        c = ck.fill_int(ck.DT_F32, (M, N), 63, 2, -3, 3)
+        want = (G.as_f64(is_bf, a) @ G.as_f64(is_bf, bt).T - 2.0 * c).astype(np.float32)   # |.| <= 192 + 6: exact in 16 bits
+        dc = torch.from_numpy(c).to(tdt).cuda()
+        da, db = G.to_dev(a), G.to_dev(bt)
+        for width in (0, 2):
+            prev = ck.set_option(ck.OPT_HALF_WIDTH, width)
+            try:
+                for cus in (256, 3):
+                    t = _straight_line_tuning(ck, cus)
+                    dd = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+                    ck.gemm_shmem_tc_async_opt_port_lp(dt, da, db, dc, dd, 1.0, -2.0, M, N, K, t["tile_dim"], t["segment_dim_k"],
+                                                       t["bar_steps_a"], t["bar_steps_b"], t["bar_step_rows_a"], t["bar_step_rows_b"],
+                                                       t["tile_group_m"], t["num_stages"], t["num_producer_warps"],
+                                                       t["num_consumer_warps"], t["num_sms"])
+                    assert ck.device_status() == 0
+                    assert np.array_equal(dd.float().cpu().numpy(), want), (dt, width, cus)
+            finally:
+                ck.set_option(ck.OPT_HALF_WIDTH, prev)
+
+
 def test_half_width_tiles_chosen_for_100_tiles_full_size(ck, oracle):
     # 2560^3: 100 tiles of 256 x 256 on 256 CUs; the launcher takes 256 x 128 tiles by itself. Whole matrix against the oracle.
     M = N = K = 2560
