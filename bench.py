@@ -248,6 +248,9 @@ def main():
     ap.add_argument("--consumers", type=int, default=None)
     ap.add_argument("--group", type=int, default=4)
     ap.add_argument("--mode", default="tile", choices=["tile", "wave", "acc"])
+    ap.add_argument("--beta", type=float, default=0.0,
+                    help="GEMM workloads: D = A Bt^T + beta C with a seeded fp32 C (the reference's own performance driver runs alpha = beta = 1, "
+                         "port_2.cu:1559-1564); default 0: no C, as the configurations are stated")
     ap.add_argument("--bar-steps-a", type=int, default=0)
     ap.add_argument("--bar-steps-b", type=int, default=0)
     ap.add_argument("--cus", type=int, default=0, help="persistent grid size (default: all compute units)")
@@ -355,8 +358,11 @@ def main():
         elif args.mode == "acc":
             rows_a = rows_b = 16
 
+        c_host = ck.fill_uniform(ck.DT_F32, (M, N), seed, 2, -1.0, 1.0) if args.beta != 0.0 else None
+        dc = None if c_host is None else torch.from_numpy(c_host).to(dev)
+
         def step():
-            ck.gemm_shmem_tc_async_opt_port(ckdt, da, db, None, dd, 1.0, 0.0, M, N, K, args.tile, args.segk,
+            ck.gemm_shmem_tc_async_opt_port(ckdt, da, db, dc, dd, 1.0, args.beta, M, N, K, args.tile, args.segk,
                                             args.bar_steps_a, args.bar_steps_b, rows_a, rows_b, args.group, args.stages,
                                             args.producers, args.consumers, cus, stream)
         peak, bound_name, arith = PEAK_TFLOPS["mfma_f16"], "mfma", dtype
@@ -456,7 +462,7 @@ def main():
         nbad, worst, nrows = 0, 0.0, 0
         for r0, r1 in row_sets:
             if kind == "gemm":
-                ref = o.gemm(o.DT_F16 if dtype == "f16" else o.DT_BF16, a, b, rows=(r0, r1))
+                ref = o.gemm(o.DT_F16 if dtype == "f16" else o.DT_BF16, a, b, c_host, 1.0, args.beta, rows=(r0, r1))
                 nb_, w_ = o.count_outside_rel(ref, got[r0:r1], 1e-2)
             else:
                 ref = o.matmul(o.DT_F32, a, b, True, False, rows=(r0, r1))
@@ -516,7 +522,7 @@ def main():
         except (RuntimeError, OSError) as e:
             out["roofline"]["measured_ceiling"] = None
             print("ceiling probe not run: %s" % e, file=sys.stderr)
-    if kind == "gemm" and args.workload == "config3_fp16_8192" and not args.no_vendor:
+    if kind == "gemm" and args.workload == "config3_fp16_8192" and not args.no_vendor and args.beta == 0.0:
         # for orientation, outside the timed region: the vendor library's kernel for the same product on the same operands
         # (fp16 in, fp32 out), timed the same way right after ours, i.e. at the same sustained clock
         try:
@@ -538,6 +544,8 @@ def main():
             out["vendor_library"] = {"error": repr(e)[:200]}
     if options:
         out["config"]["options"] = options
+    if kind == "gemm" and args.beta != 0.0:
+        out["config"]["beta"] = args.beta
     if check is not None:
         out["parity_check"] = check
     if not args.no_cpu_baseline:
