@@ -240,6 +240,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="config3_fp16_8192", choices=sorted(WORKLOADS))
+    ap.add_argument("--shape", default=None, metavar="M,N,K",
+                    help="an fp16 GEMM of this shape (uniform[-1,1) inputs) instead of a named workload, e.g. 2560,2560,2560")
     # tuning flags default to the best measured tuple of the workload (TUNED below)
     ap.add_argument("--tile", type=int, default=None)
     ap.add_argument("--segk", type=int, default=None)
@@ -322,6 +324,10 @@ def main():
     if args.grid:
         return grid(ck, torch, cus, torch.cuda.current_stream())
 
+    if args.shape:
+        sm, sn, sk = (int(v) for v in args.shape.split(","))
+        args.workload = "shape_fp16_%dx%dx%d" % (sm, sn, sk)
+        WORKLOADS[args.workload] = ("gemm", "f16", sm, sn, sk, "uniform")
     kind, dtype, M, N, K, dist = WORKLOADS[args.workload]
     # tuning flags default to what the library suggests for the shape (ckopt_suggest_gemm_tuning); TUNED records
     # what that is for the named workloads and is checked against it
@@ -332,7 +338,7 @@ def main():
     for name, val in zip(("tile", "segk", "stages", "producers", "consumers"), tuned):
         if getattr(args, name) is None:
             setattr(args, name, val)
-    seed = 0xC0FFEE00 + int(args.workload[6])
+    seed = 0xC0FFEE00 + (7 if args.shape else int(args.workload[6]))
     ckdt = {"f16": ck.DT_F16, "bf16": ck.DT_BF16, "f32": ck.DT_F32}[dtype]
     if dist == "uniform":
         a = ck.fill_uniform(ckdt, (M, K), seed, 0, -1.0, 1.0)
@@ -369,6 +375,9 @@ def main():
         if (args.producers == 0 and args.tile == 256 and args.segk == 32 and args.stages == 5 and args.consumers == 8
                 and options.get(6, 1) and options.get(0, 1)):
             kernel = "gemm_stream_kernel<%s, tile 256, five 32-deep quarters, 8 waves, pair fetch>" % dtype
+            if ck.gemm_workspace_bytes(M, N, K, True, args.tile, args.segk, args.bar_steps_a, args.bar_steps_b, rows_a, rows_b, args.group,
+                                       args.stages, args.producers, args.consumers, cus) > 0 and K % 8 == 0:
+                kernel += " with K in slices and a reduction pass"
         elif args.producers == 0:
             kernel = "gemm_fused_kernel<%s, tile %d, seg_k %d, %d waves, workgroup barrier per segment>" % (
                 dtype, args.tile, args.segk, args.consumers)
