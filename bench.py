@@ -531,11 +531,11 @@ def main():
         except (RuntimeError, OSError) as e:
             out["roofline"]["measured_ceiling"] = None
             print("ceiling probe not run: %s" % e, file=sys.stderr)
-    if kind == "gemm" and args.workload == "config3_fp16_8192" and not args.no_vendor and args.beta == 0.0:
+    if kind == "gemm" and not args.no_vendor and args.beta == 0.0:
         # for orientation, outside the timed region: the vendor library's kernel for the same product on the same operands
         # (fp16 in, fp32 out), timed the same way right after ours, i.e. at the same sustained clock
         try:
-            ta, tb = da, db.t()
+            ta, tb = (da, db.t()) if dtype == "f16" else (da.view(torch.bfloat16), db.view(torch.bfloat16).t())
             for _ in range(100):   # the other kernel draws different power: let the clock find its level again
                 torch.mm(ta, tb, out_dtype=torch.float32)
             vev0, vev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
