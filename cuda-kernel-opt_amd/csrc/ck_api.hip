@@ -417,9 +417,9 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         const StreamPlan plan = stream_plan(M, N, K, t.num_cus);
         int slices = plan.slices;
         const bool half = plan.half_width;
-        const int64_t tiles = plan.tiles;
+        const int64_t stream_tiles = plan.tiles;   // tiles of the chosen width
         if (half) a.tiles_n = (N + 127) / 128;
-        const int grid = persistent_grid(tiles, t.num_cus, a.num_xcd, g_even_rounds.load() != 0);
+        const int stream_grid = persistent_grid(stream_tiles, t.num_cus, a.num_xcd, g_even_rounds.load() != 0);
         const long long count = (long long)M * N;
         float* ws = nullptr;
         if (slices > 1) {
@@ -430,16 +430,16 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
             if (trc != CK_OK) slices = 1;
         }
         if (slices == 1) {
-            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(grid), s, a, bek, half) : launch_gemm_stream_bf16(dim3(grid), s, a, bek, half);
+            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(stream_grid), s, a, bek, half) : launch_gemm_stream_bf16(dim3(stream_grid), s, a, bek, half);
         } else {
             GemmArgs p = a;
             p.split_k = slices;
             // items are dealt slice by slice in runs of split_chunk tiles: 32 (what an XCD runs at a time) when the tiles
             // come in whole runs of 32, otherwise all tiles of a slice in one run
-            p.split_chunk = tiles % 32 == 0 ? 32 : (int)tiles;
+            p.split_chunk = stream_tiles % 32 == 0 ? 32 : (int)stream_tiles;
             p.D = ws; p.C = nullptr; p.alpha = 1.f; p.beta = 0.f; p.out16 = 0; p.vec_store = 1;
             p.nt_store = store_policy == 1 || (store_policy == 0 && whole_lines(ws, (int64_t)N * 4) && count * 4 % LINE_BYTES == 0);
-            const int64_t items = tiles * slices;
+            const int64_t items = stream_tiles * slices;
             const int pgrid = (int)(items < t.num_cus ? items : t.num_cus);
             e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p, bek, half) : launch_gemm_stream_bf16(dim3(pgrid), s, p, bek, half);
             if (e == hipSuccess) {
