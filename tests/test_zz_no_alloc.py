@@ -110,3 +110,33 @@ def test_no_alloc_entry_leaves_free_device_memory_unchanged(ck):
         assert free1 == free0
     finally:
         ck.set_option(ck.OPT_SPLIT_K, prev)
+
+
+@pytest.mark.parametrize("M,N,K", [(700, 520, 1031), (1024, 1024, 8192)])
+def test_no_alloc_entry_in_a_captured_graph(ck, M, N, K):
+    """What the entry point is for: a launch recorded into a HIP graph (operand copies for the odd K, K slices and the
+    reduction pass for the few tiles - kernels only, nothing allocated, nothing cleared by a memset node) and replayed
+    several times with eager work and synchronisations between the replays; every replay exact on small integers."""
+    t = G.tuning(**STRAIGHT_LINE)
+    order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b",
+                            "tile_group_m", "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
+    a = ck.fill_int(ck.DT_F16, (M, K), 31, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 31, 1, -2, 2)
+    exact = (a.astype(np.float64) @ bt.astype(np.float64).T).astype(np.float32)
+    da, db = G.to_dev(a), G.to_dev(bt)
+    dd = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):   # a first eager call: kernel attributes and the array's address are looked up outside the capture
+        ck.gemm_shmem_tc_async_opt_port_noalloc(ck.DT_F16, da, db, None, dd, 1.0, 0.0, M, N, K, *order, side)
+    side.synchronize()
+    assert np.array_equal(dd.cpu().numpy(), exact)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ck.gemm_shmem_tc_async_opt_port_noalloc(ck.DT_F16, da, db, None, dd, 1.0, 0.0, M, N, K, *order, torch.cuda.current_stream())
+    for replay in range(3):
+        dd.fill_(float("nan"))          # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(dd.cpu().numpy(), exact), replay
+    assert ck.device_status() == 0
