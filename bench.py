@@ -374,10 +374,14 @@ def main():
         peak, bound_name, arith = PEAK_TFLOPS["mfma_f16"], "mfma", dtype
         if (args.producers == 0 and args.tile == 256 and args.segk == 32 and args.stages == 5 and args.consumers == 8
                 and options.get(6, 1) and options.get(0, 1)):
-            kernel = "gemm_stream_kernel<%s, tile 256, five 32-deep quarters, 8 waves, pair fetch>" % dtype
-            if ck.gemm_workspace_bytes(M, N, K, True, args.tile, args.segk, args.bar_steps_a, args.bar_steps_b, rows_a, rows_b, args.group,
-                                       args.stages, args.producers, args.consumers, cus) > 0 and K % 8 == 0:
-                kernel += " with K in slices and a reduction pass"
+            plan = ck.gemm_launch_plan(M, N, K, True, args.tile, args.segk, args.bar_steps_a, args.bar_steps_b, rows_a, rows_b, args.group,
+                                       args.stages, args.producers, args.consumers, cus)
+            kernel = "gemm_stream_kernel<%s, tile %s, five 32-deep quarters, 8 waves, pair fetch>" % (
+                dtype, "256" if plan["tile_cols"] == 256 else "256 x 128")
+            if plan["k_slices"] > 1:
+                kernel += " with K in %d slices and a reduction pass" % plan["k_slices"]
+            if plan["operand_copies"]:
+                kernel += " behind zero-padded operand copies"
         elif args.producers == 0:
             kernel = "gemm_fused_kernel<%s, tile %d, seg_k %d, %d waves, workgroup barrier per segment>" % (
                 dtype, args.tile, args.segk, args.consumers)

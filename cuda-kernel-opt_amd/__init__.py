@@ -37,6 +37,8 @@ _lib.ckopt_gemm_shmem_tc_async_opt_port_2_noalloc.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_noalloc.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p]
 _lib.ckopt_gemm_workspace_bytes.restype = _i64
 _lib.ckopt_gemm_workspace_bytes.argtypes = [_i] * 15
+_lib.ckopt_gemm_launch_plan.restype = _i
+_lib.ckopt_gemm_launch_plan.argtypes = [_i] * 15 + [ctypes.POINTER(ctypes.c_int)]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_ws.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_ws.argtypes = [_i, _i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p, ctypes.c_size_t, _p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_1.restype = _i
@@ -80,7 +82,7 @@ _lib.ckopt_error_string.argtypes = [_i]
 
 EXPORTED_SYMBOLS = [
     "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_2_lp", "ckopt_gemm_shmem_tc_async_opt_port_2_noalloc",
-    "ckopt_gemm_workspace_bytes", "ckopt_gemm_shmem_tc_async_opt_port_2_ws",
+    "ckopt_gemm_workspace_bytes", "ckopt_gemm_launch_plan", "ckopt_gemm_shmem_tc_async_opt_port_2_ws",
     "ckopt_gemm_shmem_tc_async_opt_port_1",
     "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
@@ -189,6 +191,16 @@ def gemm_workspace_bytes(M, N, K, operands_aligned, tile_dim, segment_dim_k, bar
     if r < 0:
         raise CkoptError(int(r), "gemm_workspace_bytes")
     return int(r)
+
+
+def gemm_launch_plan(M, N, K, operands_aligned, tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
+                     bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms):
+    """What the launch will run: dict(straight_line, tile_cols, k_slices, operand_copies)."""
+    out = (ctypes.c_int * 4)()
+    _check(_lib.ckopt_gemm_launch_plan(M, N, K, int(bool(operands_aligned)), tile_dim, segment_dim_k, bar_steps_a, bar_steps_b,
+                                       bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+                                       num_consumer_warps, num_sms, out), "gemm_launch_plan")
+    return dict(straight_line=bool(out[0]), tile_cols=int(out[1]), k_slices=int(out[2]), operand_copies=bool(out[3]))
 
 
 def gemm_shmem_tc_async_opt_port_ws(dtype, cd_dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,

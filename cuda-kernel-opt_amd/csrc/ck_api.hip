@@ -532,6 +532,27 @@ int64_t ckopt_gemm_workspace_bytes(int M, int N, int K, int operands_aligned, in
     return need ? (int64_t)(need + SCRATCH_ALIGN) : 0;  // room to start on a 256-byte boundary inside any buffer
 }
 
+int ckopt_gemm_launch_plan(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b,
+                           int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages, int num_producer_waves,
+                           int num_consumer_waves, int num_cus, int* plan_out) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+    if (!plan_out) return ck::CK_ERR_NULL;
+    if (M <= 0 || N <= 0 || K <= 0) return ck::CK_ERR_BAD_PARAM;
+    const int rc = ck::check_gemm_tuning(t);
+    if (rc != ck::CK_OK) return rc;
+    const bool copies = K % ck::CHUNK_ELEMS != 0 || !operands_aligned;
+    const int k = copies ? padded_k(K, t) : K;
+    plan_out[0] = 0; plan_out[1] = t.tile_dim; plan_out[2] = 1; plan_out[3] = copies ? 1 : 0;
+    if (straight_line_tuple(t)) {
+        const StreamPlan plan = stream_plan(M, N, k, t.num_cus);
+        plan_out[0] = 1;
+        plan_out[1] = plan.half_width ? 128 : 256;
+        plan_out[2] = plan.slices;
+    }
+    return ck::CK_OK;
+}
+
 int ckopt_gemm_shmem_tc_async_opt_port_2_ws(int dtype, int cd_dtype, const void* A, const void* Bt, const void* C, void* D,
                                             float alpha, float beta, int M, int N, int K, int tile_dim, int segment_dim_k,
                                             int bar_steps_a, int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b,

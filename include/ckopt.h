@@ -84,6 +84,15 @@ int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void
 int64_t ckopt_gemm_workspace_bytes(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a,
                                    int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
                                    int num_producer_waves, int num_consumer_waves, int num_cus);
+
+/* What a launch with these sizes and this tuning will run under the process's current options, without launching:
+ * plan_out[0] = 1 if it takes the straight-line kernel (gemm_stream_kernel), 0 for the other designs;
+ * plan_out[1] = width of its tiles in columns of D (256 or 128 for the straight-line kernel, else tile_dim);
+ * plan_out[2] = number of K slices (1: no split-K); plan_out[3] = 1 if A and Bt are first copied into zero-padded rows.
+ * Returns CKOPT_OK or the error the launch would give. No reference counterpart (its launcher has one kernel form). */
+int ckopt_gemm_launch_plan(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b,
+                           int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages, int num_producer_waves,
+                           int num_consumer_waves, int num_cus, int* plan_out);
 int ckopt_gemm_shmem_tc_async_opt_port_2_ws(int dtype, int cd_dtype, const void* A, const void* Bt, const void* C, void* D,
                                             float alpha, float beta, int M, int N, int K, int tile_dim, int segment_dim_k,
                                             int bar_steps_a, int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b,

@@ -314,6 +314,29 @@ def test_workspace_query_follows_the_launcher_rules(ck):
             ck.gemm_workspace_bytes(*bad, True, *straight)
 
 
+def test_launch_plan_reports_what_a_launch_will_run(ck):
+    # pure host arithmetic: kernel form, tile width, K slices, operand copies - the launcher's own rules
+    straight = (256, 32, 0, 0, 256, 256, 4, 5, 0, 8, 256)
+    pc = (128, 64, 0, 0, 128, 128, 4, 2, 2, 4, 256)
+    assert ck.gemm_launch_plan(8192, 8192, 8192, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=1, operand_copies=False)
+    assert ck.gemm_launch_plan(2048, 2048, 32768, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=4, operand_copies=False)
+    assert ck.gemm_launch_plan(6143, 4097, 3071, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=1, operand_copies=True)
+    assert ck.gemm_launch_plan(2560, 2560, 2560, True, *straight) == dict(straight_line=True, tile_cols=128, k_slices=1, operand_copies=False)
+    assert ck.gemm_launch_plan(8192, 8192, 8192, False, *pc) == dict(straight_line=False, tile_cols=128, k_slices=1, operand_copies=True)
+    prev = ck.set_option(ck.OPT_HALF_WIDTH, 0)
+    try:
+        assert ck.gemm_launch_plan(2560, 2560, 2560, True, *straight)["tile_cols"] == 256
+    finally:
+        ck.set_option(ck.OPT_HALF_WIDTH, prev)
+    prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
+    try:
+        assert ck.gemm_launch_plan(8192, 8192, 8192, True, *straight)["straight_line"] is False
+    finally:
+        ck.set_option(ck.OPT_STRAIGHT_LINE, prev)
+    with pytest.raises(ck.CkoptError):
+        ck.gemm_launch_plan(0, 1, 1, True, *straight)
+
+
 def test_bench_refuses_more_than_one_gpu():
     # every box of this build has one GPU and the GEMM path has no collective: --gpus 2 exits with a message that says so
     import subprocess
