@@ -143,6 +143,20 @@ inline Tuning suggest_gemm_tuning(int M, int N, int K, int num_sms) {
     return Tuning{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9]};
 }
 
+// what a launch of `t` on these sizes will run (ckopt_gemm_launch_plan)
+struct LaunchPlan {
+    bool straight_line;
+    int tile_cols, k_slices;
+    bool operand_copies;
+};
+inline LaunchPlan gemm_launch_plan(int M, int N, int K, bool operands_aligned, const Tuning& t, int num_sms) {
+    int v[4];
+    check(ckopt_gemm_launch_plan(M, N, K, operands_aligned ? 1 : 0, t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b, t.bar_step_rows_a,
+                                 t.bar_step_rows_b, t.tile_group_m, t.num_stages, t.num_producer_warps, t.num_consumer_warps, num_sms, v),
+          "gemm_launch_plan");
+    return LaunchPlan{v[0] != 0, v[1], v[2], v[3] != 0};
+}
+
 inline int get_num_acc(int tile_dim, int num_consumer_warps) {
     const int r = ckopt_get_num_acc(tile_dim, num_consumer_warps);
     if (r < 0) throw Error(r, "get_num_acc");
