@@ -24,9 +24,9 @@
 // ODD_ONLY (an option, not the default) drops the even k-step's barrier: all four pairs of a body are
 // then issued in the odd k-step, behind its barrier (by then quarter q is free as well), and the odd
 // k-step waits for all of the wave's loads. That leaves the loads two k-steps instead of three and
-// bunches them: 1.5 % faster at 8192^3 on random operands (the device is power-limited there and holds
-// a higher clock with fewer synchronisation points), but slower wherever the loads take longer
-// (16384^3: 7 %, split-K items: 12 %) or the clock is fixed (all-zero operands: 3 %).
+// bunches them: at 8192^3 on random operands 1.5 % faster on one device and 0.7 % slower on another, and
+// slower wherever the loads take longer (16384^3: 7 %, split-K items: 6 to 12 %), the clock is free
+// (all-zero operands: 3 %) or the tiles are 256 x 128 (4 to 13 %).
 // The stream of k-steps runs across the tiles of the persistent workgroup; the loader moves to the
 // next tile two bodies before the multiplier does, so its first quarters are in flight while the
 // current tile is finished and written out.

@@ -204,8 +204,8 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  *        slice order and applies alpha, beta and the output type. 0: never. 2..16: that many slices whenever legal.
  * key 8: schedule of the straight-line kernel. 1 (default): a workgroup barrier in every k-step, the loads of a loop
  *        body spread over both (three k-steps to land); 0: one barrier per two k-steps, all loads behind it (two
- *        k-steps to land) - 1.5 % faster at 8192^3 on random operand values (power-limited clock), slower wherever
- *        memory latency is higher (16384^3: 7 %, split-K: 12 %) or the clock is not power-limited (3 %).
+ *        k-steps to land) - at 8192^3 on random operand values 1.5 % faster on one device and 0.7 % slower on another,
+ *        slower wherever memory latency is higher (16384^3: 7 %, split-K: 6 to 12 %) or the clock is free (3 %).
  * key 9: even rounds (default 1). A launch with more tiles than num_sms runs ceil(tiles / num_sms) rounds; with 1 the
  *        persistent grid is the smallest number of workgroups (a multiple of the XCD count, at most num_sms) that
  *        needs no more rounds, so that no round is partly empty (408 tiles on 256 CUs: 208 workgroups x 2 rounds
