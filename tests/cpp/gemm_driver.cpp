@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <type_traits>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -136,11 +137,53 @@ static int accuracy_shape(int M, int N, int K, int stride, int cus) {
     return failed;
 }
 
+// The <DT, DT> instance (port_2.cu:968-1055, run by the reference's main at :1519, :1533, :1545, :1559): C and D in the
+// operands' 16-bit type, alpha = beta = 1. Checked against the fp32 oracle on the same operands; the bound is the
+// reference's 0.1 plus one 16-bit rounding of a result of that size (sums of K products of uniform[-1,1) values).
+template <typename T>
+static int accuracy_shape_16_bit_cd(int M, int N, int K, int stride, int cus, float atol) {
+    const int dtype = ckopt::dtype_of<T>::value;
+    std::vector<T> a((size_t)M * K), b((size_t)N * K), c16((size_t)M * N), res((size_t)M * N);
+    std::vector<float> c((size_t)M * N), ref((size_t)M * N);
+    ckopt::check(ckopt_fill_uniform(dtype, a.data(), (int64_t)a.size(), 79, 0, -1.f, 1.f), "fill");
+    ckopt::check(ckopt_fill_uniform(dtype, b.data(), (int64_t)b.size(), 79, 1, -1.f, 1.f), "fill");
+    ckopt::check(ckopt_fill_uniform(dtype, c16.data(), (int64_t)c16.size(), 79, 2, -1.f, 1.f), "fill");
+    for (size_t i = 0; i < c.size(); ++i) c[i] = ckopt::to_float(c16[i]);
+    if (oracle_gemm_blocked(dtype, (const uint16_t*)a.data(), (const uint16_t*)b.data(), c.data(), ref.data(), 1.f, 1.f, M, N, K, 0, M, 0) != 0) return 1;
+    T *dA = nullptr, *dB = nullptr, *dC = nullptr, *dD = nullptr;
+    HIP_OK(hipMalloc((void**)&dA, a.size() * sizeof(T))); HIP_OK(hipMalloc((void**)&dB, b.size() * sizeof(T)));
+    HIP_OK(hipMalloc((void**)&dC, c16.size() * sizeof(T))); HIP_OK(hipMalloc((void**)&dD, c16.size() * sizeof(T)));
+    HIP_OK(hipMemcpy(dA, a.data(), a.size() * sizeof(T), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dB, b.data(), b.size() * sizeof(T), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dC, c16.data(), c16.size() * sizeof(T), hipMemcpyHostToDevice));
+    T one;
+    if constexpr (std::is_same<T, ckopt::half_t>::value) one = (ckopt::half_t)1.f; else one = ckopt::bfloat16_t{0x3f80};
+    int failed = 0, run = 0;
+    for (const Tuple& t : tuples(stride)) {
+        HIP_OK(hipMemset(dD, 0xff, c16.size() * sizeof(T)));
+        ckopt::gemm_shmem_tc_async_opt_port<T, T>(dA, dB, dC, dD, one, one, M, N, K, t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b,
+                                                  t.rows_a, t.rows_b, t.tile_group_m, t.num_stages, t.producers, t.consumers, cus);
+        HIP_OK(hipMemcpy(res.data(), dD, c16.size() * sizeof(T), hipMemcpyDeviceToHost));
+        long long bad = 0;
+        for (size_t i = 0; i < res.size(); ++i) bad += !(std::fabs(ckopt::to_float(res[i]) - ref[i]) <= atol);
+        ++run;
+        if (bad != 0 || ckopt_device_status(nullptr) != 0) { ++failed; print_tuple(t); std::printf(": %lld incorrect\n", bad); }
+    }
+    (void)hipFree(dA); (void)hipFree(dB); (void)hipFree(dC); (void)hipFree(dD);
+    std::printf("accuracy: <%s, %s> %d x %d x %d, %d tuples, %d with incorrect elements\n", dtype == CKOPT_DT_F16 ? "fp16" : "bf16",
+                dtype == CKOPT_DT_F16 ? "fp16" : "bf16", M, N, K, run, failed);
+    return failed;
+}
+
 static int accuracy(int cus) {
     int failed = accuracy_shape<ckopt::half_t>(512, 512, 512, 23, cus);        // the reference's own accuracy size
     failed += accuracy_shape<ckopt::bfloat16_t>(512, 512, 512, 41, cus);
     failed += accuracy_shape<ckopt::half_t>(500, 392, 520, 41, cus);           // ragged in every dimension, K not a multiple of 64
     failed += accuracy_shape<ckopt::bfloat16_t>(333, 257, 1001, 67, cus);      // rows off 16-byte boundaries: zero-padded copies
+    // results reach about 60 in magnitude: one fp16 rounding there is at most 0.016, one bf16 rounding 0.125
+    failed += accuracy_shape_16_bit_cd<ckopt::half_t>(512, 512, 512, 29, cus, 0.1f + 0.016f);
+    failed += accuracy_shape_16_bit_cd<ckopt::bfloat16_t>(512, 512, 512, 43, cus, 0.1f + 0.125f);
+    failed += accuracy_shape_16_bit_cd<ckopt::half_t>(500, 392, 520, 47, cus, 0.1f + 0.016f);
     return failed;
 }
 
