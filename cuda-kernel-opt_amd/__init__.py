@@ -19,6 +19,8 @@ DT_F16, DT_BF16, DT_F32, DT_I32 = 0, 1, 2, 3
 OK, ERR_BAD_PARAM, ERR_LDS_BUDGET, ERR_NO_INSTANCE, ERR_HIP, ERR_ALIGNMENT, ERR_NULL, ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6, -7
 OPT_SWIZZLE, OPT_SPIN_LIMIT, OPT_NUM_XCD, OPT_PRIO_MODE, OPT_PRODUCER_NAP, OPT_TILE_SYNC_BARRIER, OPT_STRAIGHT_LINE, OPT_SPLIT_K, OPT_BARRIER_EVERY_KSTEP = 0, 1, 2, 3, 4, 5, 6, 7, 8
 OPT_EVEN_ROUNDS = 9
+OPT_TAIL_ROUND = 12       # the partly filled last round of the straight-line kernel as K-sliced items of the same launch (default 1)
+OPT_FUSED_REDUCTION = 13  # 2 to 4 K slices are added inside the straight-line kernel (default 1); 0: by a second kernel
 OPT_HALF_WIDTH = 11  # 256 x 128 tiles of the straight-line kernel: 0 never, 1 where the cost model prefers them (default), 2 always
 OPT_D_STORE_POLICY = 10  # 0: non-temporal stores of D where its rows lie on 128-byte lines (default), 1: always, 2: never
 
@@ -39,6 +41,27 @@ _lib.ckopt_gemm_workspace_bytes.restype = _i64
 _lib.ckopt_gemm_workspace_bytes.argtypes = [_i] * 15
 _lib.ckopt_gemm_launch_plan.restype = _i
 _lib.ckopt_gemm_launch_plan.argtypes = [_i] * 15 + [ctypes.POINTER(ctypes.c_int)]
+
+
+class LaunchOptions(ctypes.Structure):
+    """ckopt_launch_options: the launch options as a per-call argument (fields = the ckopt_set_option keys in order)."""
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "struct_bytes", "lds_swizzle", "spin_limit", "num_xcd", "prio_mode", "producer_nap", "tile_sync_barrier", "straight_line",
+        "split_k", "barrier_every_kstep", "even_rounds", "d_store_policy", "half_width", "tail_round", "fused_reduction")]
+
+
+_lib.ckopt_launch_options_init.restype = _i
+_lib.ckopt_launch_options_init.argtypes = [ctypes.POINTER(LaunchOptions)]
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2_ex.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_2_ex.argtypes = [_i, _i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [ctypes.POINTER(LaunchOptions), _p, ctypes.c_size_t, _p]
+_lib.ckopt_gemm_workspace_bytes_ex.restype = _i64
+_lib.ckopt_gemm_workspace_bytes_ex.argtypes = [_i] * 15 + [ctypes.POINTER(LaunchOptions)]
+_lib.ckopt_gemm_launch_plan_ex.restype = _i
+_lib.ckopt_gemm_launch_plan_ex.argtypes = [_i] * 15 + [ctypes.POINTER(LaunchOptions), ctypes.POINTER(ctypes.c_int)]
+_lib.ckopt_gemm_shmem_tc_async_opt_port_1_lp.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_1_lp.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 12 + [_p]
+_lib.ckopt_gemm_shmem_tc_async_opt_port_0_lp.restype = _i
+_lib.ckopt_gemm_shmem_tc_async_opt_port_0_lp.argtypes = [_i, _p, _p, _p, _p, _f, _f] + [_i] * 10 + [_p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_ws.restype = _i
 _lib.ckopt_gemm_shmem_tc_async_opt_port_2_ws.argtypes = [_i, _i, _p, _p, _p, _p, _f, _f] + [_i] * 14 + [_p, ctypes.c_size_t, _p]
 _lib.ckopt_gemm_shmem_tc_async_opt_port_1.restype = _i
@@ -83,8 +106,9 @@ _lib.ckopt_error_string.argtypes = [_i]
 EXPORTED_SYMBOLS = [
     "ckopt_gemm_shmem_tc_async_opt_port_2", "ckopt_gemm_shmem_tc_async_opt_port_2_lp", "ckopt_gemm_shmem_tc_async_opt_port_2_noalloc",
     "ckopt_gemm_workspace_bytes", "ckopt_gemm_launch_plan", "ckopt_gemm_shmem_tc_async_opt_port_2_ws",
-    "ckopt_gemm_shmem_tc_async_opt_port_1",
-    "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
+    "ckopt_launch_options_init", "ckopt_gemm_shmem_tc_async_opt_port_2_ex", "ckopt_gemm_workspace_bytes_ex", "ckopt_gemm_launch_plan_ex",
+    "ckopt_gemm_shmem_tc_async_opt_port_1", "ckopt_gemm_shmem_tc_async_opt_port_1_lp",
+    "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_gemm_shmem_tc_async_opt_port_0_lp", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
     "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks",
     "ckopt_suggest_gemm_tuning",
@@ -183,24 +207,52 @@ def gemm_shmem_tc_async_opt_port_lp(dtype, A, B, C, D, alpha, beta, M, N, K, til
 
 
 def gemm_workspace_bytes(M, N, K, operands_aligned, tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
-                         bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms):
-    """Bytes of caller-owned workspace gemm_shmem_tc_async_opt_port_ws needs for this launch (0: none)."""
-    r = _lib.ckopt_gemm_workspace_bytes(M, N, K, int(bool(operands_aligned)), tile_dim, segment_dim_k, bar_steps_a, bar_steps_b,
-                                        bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
-                                        num_consumer_warps, num_sms)
+                         bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, options=None):
+    """Bytes of caller-owned workspace gemm_shmem_tc_async_opt_port_ws / _ex needs for this launch (0: none)."""
+    r = _lib.ckopt_gemm_workspace_bytes_ex(M, N, K, int(bool(operands_aligned)), tile_dim, segment_dim_k, bar_steps_a, bar_steps_b,
+                                           bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+                                           num_consumer_warps, num_sms, _optr(options))
     if r < 0:
         raise CkoptError(int(r), "gemm_workspace_bytes")
     return int(r)
 
 
+def launch_options(**fields):
+    """The process-wide default options as a LaunchOptions value, with the given fields replaced."""
+    o = LaunchOptions()
+    _check(_lib.ckopt_launch_options_init(ctypes.byref(o)), "launch_options_init")
+    for k, v in fields.items():
+        if k not in dict(LaunchOptions._fields_) or k == "struct_bytes":
+            raise KeyError(k)
+        setattr(o, k, int(v))
+    return o
+
+
+def _optr(options):
+    return None if options is None else ctypes.byref(options)
+
+
 def gemm_launch_plan(M, N, K, operands_aligned, tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
-                     bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms):
-    """What the launch will run: dict(straight_line, tile_cols, k_slices, operand_copies)."""
-    out = (ctypes.c_int * 4)()
-    _check(_lib.ckopt_gemm_launch_plan(M, N, K, int(bool(operands_aligned)), tile_dim, segment_dim_k, bar_steps_a, bar_steps_b,
-                                       bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
-                                       num_consumer_warps, num_sms, out), "gemm_launch_plan")
-    return dict(straight_line=bool(out[0]), tile_cols=int(out[1]), k_slices=int(out[2]), operand_copies=bool(out[3]))
+                     bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, options=None):
+    """What the launch will run: dict(straight_line, tile_cols, k_slices, operand_copies, sliced_tiles, reduced_in_kernel, grid)."""
+    out = (ctypes.c_int * 7)()
+    _check(_lib.ckopt_gemm_launch_plan_ex(M, N, K, int(bool(operands_aligned)), tile_dim, segment_dim_k, bar_steps_a, bar_steps_b,
+                                          bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+                                          num_consumer_warps, num_sms, _optr(options), out), "gemm_launch_plan")
+    return dict(straight_line=bool(out[0]), tile_cols=int(out[1]), k_slices=int(out[2]), operand_copies=bool(out[3]),
+                sliced_tiles=int(out[4]), reduced_in_kernel=bool(out[5]), grid=int(out[6]))
+
+
+def gemm_shmem_tc_async_opt_port_ex(dtype, cd_dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+                                    bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages,
+                                    num_producer_warps, num_consumer_warps, num_sms, options=None, workspace=None, workspace_bytes=0,
+                                    stream=None):
+    """The port_2 launcher with its options as an argument (a LaunchOptions; None: the process-wide defaults) and,
+    optionally, a caller-owned workspace (None: stream-ordered allocations)."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_2_ex(
+        dtype, cd_dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
+        bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps,
+        num_sms, _optr(options), _dptr(workspace), int(workspace_bytes), _stream(stream)), "gemm_shmem_tc_async_opt_port (options)")
 
 
 def gemm_shmem_tc_async_opt_port_ws(dtype, cd_dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_steps_a,
@@ -243,6 +295,24 @@ def gemm_shmem_tc_async_opt_port_0(dtype, A, B, C, D, alpha, beta, M, N, K, tile
     _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_0(
         dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, tile_group_m,
         num_stages, num_producer_warps, num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port_0")
+
+
+def gemm_shmem_tc_async_opt_port_1_lp(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_step_rows_a,
+                                      bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps,
+                                      num_sms, stream=None):
+    """The <half, half> instance of the port_1 launcher (port_1.cu:1292, :1332): C and D in the operands' 16-bit type."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_1_lp(
+        dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_step_rows_a,
+        bar_step_rows_b, tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, _stream(stream)),
+        "gemm_shmem_tc_async_opt_port_1 <DT, DT>")
+
+
+def gemm_shmem_tc_async_opt_port_0_lp(dtype, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, tile_group_m,
+                                      num_stages, num_producer_warps, num_consumer_warps, num_sms, stream=None):
+    """The <half, half> instance of the port_0 launcher (port_0.cu:866, :906)."""
+    _check(_lib.ckopt_gemm_shmem_tc_async_opt_port_0_lp(
+        dtype, _dptr(A), _dptr(B), _dptr(C), _dptr(D), alpha, beta, M, N, K, tile_dim, segment_dim_k, tile_group_m,
+        num_stages, num_producer_warps, num_consumer_warps, num_sms, _stream(stream)), "gemm_shmem_tc_async_opt_port_0 <DT, DT>")
 
 
 def matmul_shmem(dtype, A, B, C, M, N, K, tile_dim, block_rows, b_transposed=False, stream=None):

@@ -44,19 +44,38 @@ static __device__ __align__(256) unsigned char scratch[CKOPT_NOALLOC_SCRATCH_BYT
 
 namespace {
 
-std::atomic<int> g_swizzle{1};
-std::atomic<int> g_spin_limit{1 << 22};
-std::atomic<int> g_num_xcd{8};
-std::atomic<int> g_prio_mode{0};
-std::atomic<int> g_producer_nap{0};
-std::atomic<int> g_tile_sync_barrier{0};
-std::atomic<int> g_straight_line{1};
-std::atomic<int> g_even_rounds{1};
-std::atomic<int> g_split_k{1};  // 0: never, 1: when few tiles would leave most CUs idle, >= 2: that many slices if legal
-std::atomic<int> g_barrier_every_kstep{1};
-std::atomic<int> g_half_width{1};  // 256 x 128 tiles of the straight-line kernel: 0 never, 1 where the cost model prefers them, 2 always
-std::atomic<int> g_d_store_policy{0};  // 0: non-temporal stores of D where its rows lie on 128-byte lines, 1: always, 2: never
+// The knobs that are not launcher parameters in the reference. A launch works on one Options value: the caller's
+// ckopt_launch_options, or a snapshot of the process-wide defaults taken once when the entry point starts.
+enum { OPT_SWIZZLE, OPT_SPIN_LIMIT, OPT_NUM_XCD, OPT_PRIO_MODE, OPT_PRODUCER_NAP, OPT_TILE_SYNC_BARRIER, OPT_STRAIGHT_LINE, OPT_SPLIT_K,
+       OPT_BARRIER_EVERY_KSTEP, OPT_EVEN_ROUNDS, OPT_D_STORE_POLICY, OPT_HALF_WIDTH, OPT_TAIL_ROUND, OPT_FUSED_REDUCTION, NUM_OPTIONS };
+struct OptionRule { int initial, lo, hi; };
+constexpr OptionRule OPTION_RULES[NUM_OPTIONS] = {
+    {1, 0, 1}, {1 << 22, 1, 0x7fffffff}, {8, 1, 64}, {0, 0, 2}, {0, 0, 2}, {0, 0, 1}, {1, 0, 1}, {1, 0, 16},
+    {1, 0, 1}, {1, 0, 1}, {0, 0, 2}, {1, 0, 2}, {1, 0, 1}, {1, 0, 2}};
+std::atomic<int> g_option[NUM_OPTIONS] = {{1}, {1 << 22}, {8}, {0}, {0}, {0}, {1}, {1}, {1}, {1}, {0}, {1}, {1}, {1}};
+struct Options {
+    int v[NUM_OPTIONS];
+    int operator[](int key) const { return v[key]; }
+};
+Options default_options() {
+    Options o;
+    for (int k = 0; k < NUM_OPTIONS; ++k) o.v[k] = g_option[k].load();
+    return o;
+}
+// the public struct's fields follow struct_bytes in key order
+int options_from_public(const ckopt_launch_options* p, Options* out) {
+    if (!p) { *out = default_options(); return ck::CK_OK; }
+    if (p->struct_bytes != (int)sizeof(ckopt_launch_options)) return ck::CK_ERR_BAD_PARAM;
+    const int* f = &p->lds_swizzle;
+    for (int k = 0; k < NUM_OPTIONS; ++k) {
+        if (f[k] < OPTION_RULES[k].lo || f[k] > OPTION_RULES[k].hi) return ck::CK_ERR_BAD_PARAM;
+        out->v[k] = f[k];
+    }
+    return ck::CK_OK;
+}
+static_assert(sizeof(ckopt_launch_options) == (NUM_OPTIONS + 1) * sizeof(int), "one int per key behind struct_bytes");
 constexpr int LINE_BYTES = 128;         // cache line of the vector memory path
+constexpr int TAIL_ROUND_MAX_SLICES = 4;   // the partly filled last round is cut into at most this many slices
 constexpr int SPLIT_K_MIN_SLICE = 1024;  // shortest K slice split-K will make (shorter ones lose more in the reduction pass than they gain)
 
 constexpr int MAX_DEV = 64;
@@ -78,6 +97,27 @@ int status_ptr_for_current_device(unsigned int** out) {
 }
 
 unsigned char* g_scratch_ptr[MAX_DEV] = {};
+
+// Compute units of the current device (what the cost model's measurements scale with), read once per device;
+// 256, the device the model was calibrated on, where no device can be asked.
+int g_device_cus[MAX_DEV] = {};
+int device_cus() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    std::lock_guard<std::mutex> lock(g_status_mutex);
+    if (!g_device_cus[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        g_device_cus[dev] = n;
+    }
+    return g_device_cus[dev];
+}
 
 // Device address of this device's copy of `scratch`, looked up once per device with that device current.
 int static_scratch_for_current_device(unsigned char** out) {
@@ -177,6 +217,12 @@ __global__ void splitk_reduce4_kernel(const f32x4* __restrict__ ws, int slices, 
     }
 }
 
+// Clears the arrival words of the reduction inside the straight-line kernel (a kernel, not a memset: callers may
+// record the launch into a graph).
+__global__ void zero_words_kernel(unsigned int* p, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) p[i] = 0u;
+}
+
 // Where a launch takes device memory beyond its operands from (the zero-padded operand copies, the split-K planes).
 // ALLOCATE: stream-ordered allocations inside the call. PROVIDED: the buffer [ptr, ptr + bytes) that the caller or the
 // library's static array supplies; pieces are carved off its front on 256-byte boundaries and nothing is allocated.
@@ -214,7 +260,86 @@ bool scratch_release(const Scratch& sc, void* piece, hipStream_t s) {
 }
 
 int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
-                int N, int K, const ck::GemmTuning& t, void* stream, int out16, Scratch sc);
+                int N, int K, const ck::GemmTuning& t, const Options& opt, void* stream, int out16, Scratch sc);
+
+// Estimated duration (microseconds) of the straight-line kernel on `tiles` tiles (256 x 256, or 256 x 128 with
+// half_width) of an M x N product with K cut into S slices, plus what adding the slices costs when S > 1. The constants
+// are measurements of one MI355X (256 CUs) on random operands: a loop body (64 of K) of a 256 x 256 tile takes 1.05 us
+// while at most half of the CUs multiply and the clock is free, and grows with the share of active CUs once the device is
+// power-limited (1.42 us with all of them); a 256 x 128 tile's body has half the MFMAs and takes 0.585 of that time
+// at the power-limited clock but no less than 0.69 us (one barrier per 16 MFMAs); a work item costs about 3 us of pipeline
+// fill and drain; the items of a round store their tile at the 4.6 TB/s the write path sustains. The slices are added
+// either by a reduction pass (reads S planes and writes D at 5.3 TB/s behind about 3 us of launch) or, `fused`, by the
+// last wave tile to arrive, which reads the S - 1 others at what one CU draws from memory (about 110 GB/s). device_cus is
+// the device's real CU count: the power-limit knee lies at half of it. The model is calibrated for a 256-CU gfx950.
+constexpr double HALF_WIDTH_BODY = 0.585, HALF_WIDTH_BODY_MIN_US = 0.69;
+double body_us_for(double active, bool half_width, int dev_cus) {
+    const double full_body_us = 1.05 * std::max(1.0, std::pow(active / (0.5 * dev_cus), 0.43));
+    return half_width ? std::max(HALF_WIDTH_BODY_MIN_US, HALF_WIDTH_BODY * full_body_us) : full_body_us;
+}
+// one round of `active` work items of `bodies` loop bodies each, with the store burst that ends it
+double round_us_for(double active, double bodies, bool half_width, int dev_cus) {
+    const double store_us = active * (half_width ? 128.0 : 256.0) * 1024.0 / 4.6e6;
+    return bodies * body_us_for(active, half_width, dev_cus) + store_us + 3.0;
+}
+// what adding the slices costs: inside the kernel (every wave stores the rows it does not own, waits for its S - 1
+// partners and reads what they stored for its rows; measured on config-4-like shapes: about 6 us and 12 us per further
+// slice, most of it the wait for the slowest partner - two slices of 128 tiles: 18 us against 22 for the pass; four of 64
+// tiles: 42 against 19; eight of 32 half-width tiles: 44 against 10), or by the reduction pass
+double fused_reduction_us(int S, bool half_width) { return 6.0 + (half_width ? 6.0 : 12.0) * (double)(S - 1); }
+double reduction_pass_us(int S, int64_t mn) { return 3.0 + (double)(S + 1) * (double)mn * 4.0 / 5.3e6; }
+double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus, bool half_width, bool fused, int dev_cus) {
+    const double items = (double)tiles * S;
+    const double rounds = std::ceil(items / num_cus);
+    const double active = items / rounds;   // workgroups (CUs) busy in a round
+    const double bodies = (double)K / S / ck::STREAM_K_MULTIPLE_HOST;
+    double t = rounds * round_us_for(active, bodies, half_width, dev_cus);
+    if (S > 1) t += fused ? fused_reduction_us(S, half_width) : reduction_pass_us(S, mn);
+    return t;
+}
+
+// How the straight-line kernel runs an M x N x K product on num_cus workgroups.
+struct StreamPlan {
+    bool half_width;       // 256 x 128 tiles
+    int64_t tiles;         // tiles of that width
+    int64_t whole_tiles;   // tile counts [0, whole_tiles) run over all of K ...
+    int slices;            // ... the others in this many K slices each (1: none are cut, whole_tiles == tiles)
+    bool fused;            // the slices are added inside the kernel (else by a second pass over slices x M x N planes)
+    int grid;              // workgroups
+    double us;             // the estimate that decided
+};
+
+bool slices_legal(int K, int c) { return c >= 2 && K % (c * ck::STREAM_K_MULTIPLE_HOST) == 0 && K / c >= SPLIT_K_MIN_SLICE; }
+// The slices are added inside the kernel where that is allowed - the option; the waves that hold the slices of a wave tile
+// wait for one another, so all of them must be running at once: every workgroup at most one sliced item (sliced_items <=
+// num_cus) and no more workgroups than the device has CUs - and estimated cheaper than the reduction pass.
+bool reduces_in_kernel(const Options& opt, int slices, int64_t sliced_tiles, int64_t mn, int num_cus, bool half_width, int dev_cus) {
+    if (!opt[OPT_FUSED_REDUCTION] || slices < 2 || num_cus > dev_cus || sliced_tiles * slices > num_cus) return false;
+    return opt[OPT_FUSED_REDUCTION] == 2 || fused_reduction_us(slices, half_width) < reduction_pass_us(slices, mn);
+}
+
+// Number of K slices for `tiles` tiles that all are cut (1: no split). policy 0: never; 1: automatic - with fewer tiles
+// than CUs, the legal slice count whose estimated duration is shortest (a larger count must win by 3 %: it costs scratch
+// memory); >= 2: that many slices if legal, else the next smaller legal count.
+// Legal: slices of whole loop bodies and at least SPLIT_K_MIN_SLICE deep (any tile count, any N).
+int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, const Options& opt, bool half_width, int dev_cus) {
+    const int policy = opt[OPT_SPLIT_K];
+    if (policy == 0 || tiles <= 0) return 1;
+    if (policy >= 2) {
+        int cand = policy > 16 ? 16 : policy;
+        while (cand >= 2 && !slices_legal(K, cand)) --cand;
+        return cand < 2 ? 1 : cand;
+    }
+    if (tiles >= num_cus) return 1;
+    int best = 1;
+    double best_us = split_k_estimate_us(tiles, mn, K, 1, num_cus, half_width, false, dev_cus);
+    for (int c = 2; c <= 16; ++c) {
+        if (!slices_legal(K, c)) continue;
+        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus, half_width, reduces_in_kernel(opt, c, tiles, mn, num_cus, half_width, dev_cus), dev_cus);
+        if (us < 0.97 * best_us) { best = c; best_us = us; }
+    }
+    return best;
+}
 
 // Workgroups of the persistent grid. With more tiles than CUs, num_cus workgroups run ceil(tiles / num_cus)
 // rounds and the last one is partly empty: CUs idle at the end while the full rounds before it ran at the
@@ -230,66 +355,45 @@ int persistent_grid(int64_t tiles, int num_cus, int num_xcd, bool even_rounds) {
     return (int)(g < num_cus ? g : num_cus);
 }
 
-// Estimated duration (microseconds) of the straight-line kernel on `tiles` tiles (256 x 256, or 256 x 128 with
-// half_width) of an M x N product with K cut into S slices, plus the reduction pass when S > 1. The constants are
-// measurements of one MI355X on random operands: a loop body (64 of K) of a 256 x 256 tile takes 1.05 us while at most
-// half of the 256 CUs multiply and the clock is free, and grows with the number of active CUs once the device is
-// power-limited (1.42 us with all of them); a 256 x 128 tile's body has half the MFMAs and takes 0.585 of that time
-// at the power-limited clock but no less than 0.69 us (one barrier per 16 MFMAs); a work item costs about 3 us of pipeline fill and drain; the items of a round store their tile at the
-// 4.6 TB/s the write path sustains; the reduction pass reads S planes and writes D at 5.3 TB/s behind about 3 us of launch.
-constexpr double HALF_WIDTH_BODY = 0.585, HALF_WIDTH_BODY_MIN_US = 0.69;
-double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus, bool half_width) {
-    const double items = (double)tiles * S;
-    const double rounds = std::ceil(items / num_cus);
-    const double active = items / rounds;   // workgroups (CUs) busy in a round
-    const double full_body_us = 1.05 * std::max(1.0, std::pow(active / 128.0, 0.43));
-    const double body_us = half_width ? std::max(HALF_WIDTH_BODY_MIN_US, HALF_WIDTH_BODY * full_body_us) : full_body_us;
-    const double bodies = (double)K / S / ck::STREAM_K_MULTIPLE_HOST;
-    const double store_us = active * (half_width ? 128.0 : 256.0) * 1024.0 / 4.6e6;
-    double t = rounds * (bodies * body_us + store_us + 3.0);
-    if (S > 1) t += 3.0 + (double)(S + 1) * (double)mn * 4.0 / 5.3e6;
-    return t;
-}
-
-// Number of K slices the straight-line kernel uses for `tiles` tiles (1: no split). policy 0: never;
-// 1: automatic - with fewer tiles than CUs, the legal slice count whose estimated duration is shortest (a larger count
-// must win by 3 %: it costs scratch memory); >= 2: that many slices if legal, else the next smaller legal count.
-// Legal: slices of whole loop bodies and at least SPLIT_K_MIN_SLICE deep (any tile count, any N).
-int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, int policy, bool half_width) {
-    if (policy == 0 || tiles <= 0) return 1;
-    auto legal = [&](int c) { return K % (c * ck::STREAM_K_MULTIPLE_HOST) == 0 && K / c >= SPLIT_K_MIN_SLICE; };
-    if (policy >= 2) {
-        int cand = policy > 16 ? 16 : policy;
-        while (cand >= 2 && !legal(cand)) --cand;
-        return cand < 2 ? 1 : cand;
-    }
-    if (tiles >= num_cus) return 1;
-    int best = 1;
-    double best_us = split_k_estimate_us(tiles, mn, K, 1, num_cus, half_width);
-    for (int c = 2; c <= 16; ++c) {
-        if (!legal(c)) continue;
-        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus, half_width);
-        if (us < 0.97 * best_us) { best = c; best_us = us; }
-    }
-    return best;
-}
-
-// How the straight-line kernel runs an M x N x K product on num_cus workgroups: tile width, K slices, and the
-// estimate that decided. 256 x 128 tiles where they are estimated at least 5 % faster (they fill a device that few
-// 256 x 256 tiles leave idle, at a lower rate per CU), or always / never by the option.
-struct StreamPlan {
-    bool half_width;
-    int slices;
-    int64_t tiles;
-    double us;
-};
-StreamPlan stream_plan(int M, int N, int K, int num_cus) {
+// Tile width, K slices and grid of a launch. With fewer tiles than CUs every tile may be cut (split_k_slices). With more,
+// the full rounds run whole tiles on all num_cus workgroups and the tiles of the partly filled last round are cut into 2
+// to 4 slices reduced in the kernel, in the same launch, where that is estimated at least 5 % shorter than rounds of
+// whole tiles (6144^3 measures the same either way, 391 us: 576 tiles as 2 x 256 whole tiles + 64 tiles in 2 slices, or as
+// 3 rounds of 192 whole tiles; with the 5 % margin it takes the rounds). 256 x 128 tiles where they are
+// estimated at least 5 % faster than 256 x 256 (they fill a device that few large tiles leave idle, at a lower rate per
+// CU), or always / never by the option.
+StreamPlan stream_plan(int M, int N, int K, int num_cus, const Options& opt) {
     const int64_t mn = (int64_t)M * N;
-    const int policy = g_split_k.load(), width = g_half_width.load();
+    const int width = opt[OPT_HALF_WIDTH], dev_cus = device_cus();
+    const bool even = opt[OPT_EVEN_ROUNDS] != 0;
     auto plan = [&](bool half) {
         const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + (half ? 127 : 255)) / (half ? 128 : 256));
-        const int slices = split_k_slices(tiles, mn, K, num_cus, policy, half);
-        return StreamPlan{half, slices, tiles, split_k_estimate_us(tiles, mn, K, slices, num_cus, half)};
+        StreamPlan p{half, tiles, tiles, 1, false, persistent_grid(tiles, num_cus, opt[OPT_NUM_XCD], even), 0.0};
+        if (tiles <= num_cus) {
+            p.slices = split_k_slices(tiles, mn, K, num_cus, opt, half, dev_cus);
+            p.fused = reduces_in_kernel(opt, p.slices, tiles, mn, num_cus, half, dev_cus);
+            if (p.slices > 1) {
+                p.whole_tiles = 0;
+                p.grid = (int)std::min<int64_t>(tiles * p.slices, num_cus);
+            }
+            p.us = split_k_estimate_us(tiles, mn, K, p.slices, num_cus, half, p.fused, dev_cus);
+            return p;
+        }
+        // rounds of whole tiles (as many rounds as num_cus workgroups need, evenly filled)
+        const double rounds = std::ceil((double)tiles / num_cus), bodies = (double)K / ck::STREAM_K_MULTIPLE_HOST;
+        p.us = rounds * round_us_for(even ? (double)tiles / rounds : (double)num_cus, bodies, half, dev_cus);
+        const int64_t full = tiles / num_cus * num_cus, rest = tiles - full;
+        if (rest > 0 && opt[OPT_TAIL_ROUND] && opt[OPT_FUSED_REDUCTION] && opt[OPT_SPLIT_K] == 1 && num_cus <= dev_cus) {
+            const double head_us = (double)(full / num_cus) * round_us_for(num_cus, bodies, half, dev_cus);
+            for (int c = 2; c <= TAIL_ROUND_MAX_SLICES; ++c) {
+                if (!slices_legal(K, c) || rest * c > num_cus) continue;
+                const double us = head_us + split_k_estimate_us(rest, mn, K, c, num_cus, half, true, dev_cus);
+                if (us < 0.95 * p.us) {
+                    p.us = us; p.slices = c; p.fused = true; p.whole_tiles = full; p.grid = num_cus;
+                }
+            }
+        }
+        return p;
     };
     const StreamPlan full = plan(false);
     if (width == 0) return full;
@@ -298,32 +402,46 @@ StreamPlan stream_plan(int M, int N, int K, int num_cus) {
     return half.us < 0.95 * full.us ? half : full;
 }
 
+// Scratch memory of the K slices of a plan. Reduced in the kernel: per sliced tile slices - 1 tiles of fp32 in the
+// accumulators' layout (what the slices' waves store of the rows they do not own), behind the announcement counters (one
+// 128-byte line per sliced tile and wave, cleared by every launch). Reduced by the second pass: slices planes of M x N fp32.
+constexpr size_t FIX_STATE_BYTES_PER_TILE = 8 * 128;   // eight waves, one counter per 128-byte line (FIX_STATE_STRIDE_BYTES of the kernel)
+size_t fix_state_bytes(const StreamPlan& p) { return (size_t)(p.tiles - p.whole_tiles) * FIX_STATE_BYTES_PER_TILE; }
+size_t fix_partial_bytes(const StreamPlan& p) {
+    return (size_t)(p.tiles - p.whole_tiles) * (size_t)(p.slices - 1) * 256 * (p.half_width ? 128 : 256) * sizeof(float);
+}
+
 // The tuning tuple the straight-line kernel is written for (it also needs K in whole loop bodies of 64).
-bool straight_line_tuple(const ck::GemmTuning& t) {
-    return g_straight_line.load() && g_swizzle.load() && t.num_producer_waves == 0 && t.num_consumer_waves == 8 && t.tile_dim == 256 &&
+bool straight_line_tuple(const ck::GemmTuning& t, const Options& opt) {
+    return opt[OPT_STRAIGHT_LINE] && opt[OPT_SWIZZLE] && t.num_producer_waves == 0 && t.num_consumer_waves == 8 && t.tile_dim == 256 &&
            t.segment_dim_k == 32 && t.num_stages == 5;
 }
-// K of the zero-padded operand copies (made when K % 8 != 0 or an operand is off a 16-byte boundary): whole 16-byte
-// chunks, and for the straight-line tuple whole loop bodies, so that the copies take that kernel's plain instance.
-int padded_k(int K, const ck::GemmTuning& t) {
-    const int unit = straight_line_tuple(t) ? ck::STREAM_K_MULTIPLE_HOST : ck::CHUNK_ELEMS;
+// Does a launch on these sizes first copy A and Bt into zero-padded rows, and with which K? The kernels read operand rows
+// that start on 16-byte boundaries in whole 16-byte chunks: copies are made when K % 8 != 0 or an operand is off a
+// 16-byte boundary, with K rounded up to whole chunks - for the straight-line tuple to whole loop bodies, so that the
+// copies take that kernel's plain instance.
+bool needs_copies(int K, bool operands_aligned) { return K % ck::CHUNK_ELEMS != 0 || !operands_aligned; }
+int padded_k(int K, const ck::GemmTuning& t, const Options& opt) {
+    const int unit = straight_line_tuple(t, opt) ? ck::STREAM_K_MULTIPLE_HOST : ck::CHUNK_ELEMS;
     return (K + unit - 1) / unit * unit;
+}
+// K the kernels of a launch work on (the one rule the launcher, the workspace query, the plan query and the tuning
+// suggestion share)
+int launch_k(int K, bool operands_aligned, const ck::GemmTuning& t, const Options& opt) {
+    return needs_copies(K, operands_aligned) ? padded_k(K, t, opt) : K;
 }
 
 // Scratch bytes a launch takes from a provided buffer whose start is on a 256-byte boundary (the launcher's own
-// rules, evaluated without launching): the zero-padded operand copies when K % 8 != 0 or the operands are not on
-// 16-byte boundaries, then the split-K planes when the straight-line kernel cuts K.
-size_t scratch_need(int M, int N, int K, bool operands_aligned, const ck::GemmTuning& t) {
+// rules, evaluated without launching): the zero-padded operand copies, then what the K slices need.
+size_t scratch_need(int M, int N, int K, bool operands_aligned, const ck::GemmTuning& t, const Options& opt) {
     using namespace ck;
     size_t need = 0;
-    int k = K;
-    if (K % CHUNK_ELEMS != 0 || !operands_aligned) {
-        k = padded_k(K, t);
-        need += scratch_round(((size_t)M + (size_t)N) * k * 2);
-    }
-    if (straight_line_tuple(t)) {
-        const int slices = stream_plan(M, N, k, t.num_cus).slices;
-        if (slices > 1) need += scratch_round((size_t)slices * M * N * sizeof(float));
+    const int k = launch_k(K, operands_aligned, t, opt);
+    if (needs_copies(K, operands_aligned)) need += scratch_round(((size_t)M + (size_t)N) * k * 2);
+    if (straight_line_tuple(t, opt)) {
+        const StreamPlan p = stream_plan(M, N, k, t.num_cus, opt);
+        if (p.slices > 1 && p.fused) need += scratch_round(fix_state_bytes(p)) + scratch_round(fix_partial_bytes(p));
+        else if (p.slices > 1) need += scratch_round((size_t)p.slices * M * N * sizeof(float));
     }
     return need;
 }
@@ -331,9 +449,9 @@ size_t scratch_need(int M, int N, int K, bool operands_aligned, const ck::GemmTu
 // K % 8 != 0 or operands off a 16-byte boundary: the product is computed from zero-padded,
 // aligned copies of A and Bt in a stream-ordered temporary (zeros in the K tail add nothing).
 int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta,
-                         int M, int N, int K, const ck::GemmTuning& t, void* stream, int out16, Scratch sc) {
+                         int M, int N, int K, const ck::GemmTuning& t, const Options& opt, void* stream, int out16, Scratch sc) {
     using namespace ck;
-    const int Kp = padded_k(K, t);
+    const int Kp = padded_k(K, t, opt);
     const size_t bytes_a = (size_t)M * Kp * 2, bytes_b = (size_t)N * Kp * 2;
     hipStream_t s = static_cast<hipStream_t>(stream);
     void* ws = nullptr;
@@ -346,13 +464,13 @@ int gemm_launch_repacked(int dtype, const void* A, const void* Bt, const void* C
     hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks(((long long)M + N) * (Kp / 8))), dim3(threads), 0, s, static_cast<const unsigned short*>(A), pa, M,
                        static_cast<const unsigned short*>(Bt), pb, N, K, Kp);
     int rc = hipGetLastError() == hipSuccess ? CK_OK : CK_ERR_HIP;
-    if (rc == CK_OK) rc = gemm_launch(dtype, pa, pb, C, D, alpha, beta, M, N, Kp, t, stream, out16, sc);
+    if (rc == CK_OK) rc = gemm_launch(dtype, pa, pb, C, D, alpha, beta, M, N, Kp, t, opt, stream, out16, sc);
     if (!scratch_release(sc, ws, s) && rc == CK_OK) rc = CK_ERR_HIP;
     return rc;
 }
 
 int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
-                int N, int K, const ck::GemmTuning& t, void* stream, int out16, Scratch sc) {
+                int N, int K, const ck::GemmTuning& t, const Options& opt, void* stream, int out16, Scratch sc) {
     using namespace ck;
     if (!(dtype == CK_DT_F16 || dtype == CK_DT_BF16)) return CK_ERR_BAD_PARAM;
     if (M <= 0 || N <= 0 || K <= 0) return CK_ERR_BAD_PARAM;
@@ -364,8 +482,8 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     const uintptr_t elem_mask = out16 ? 1 : 3;
     if (((uintptr_t)D & elem_mask) || ((uintptr_t)C & elem_mask)) return CK_ERR_ALIGNMENT;
     // the kernels want every operand row on a 16-byte boundary
-    if (K % CHUNK_ELEMS != 0 || ((uintptr_t)A & 15) || ((uintptr_t)Bt & 15))
-        return gemm_launch_repacked(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, out16, sc);
+    if (needs_copies(K, !(((uintptr_t)A | (uintptr_t)Bt) & 15)))
+        return gemm_launch_repacked(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, opt, stream, out16, sc);
     // one tile's rows are addressed through a 32-bit buffer offset
     if ((int64_t)t.tile_dim * K * 2 >= (int64_t)1 << 31) return CK_ERR_TOO_LARGE;
 
@@ -380,71 +498,103 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     a.nseg = (K + t.segment_dim_k - 1) / t.segment_dim_k;
     a.tile_group_m = t.tile_group_m;
     a.num_stages = t.num_stages;
-    a.pa = t.num_producer_waves / 2;
-    a.pb = t.num_producer_waves - a.pa;
+    // one producer wave (port_0 only): it streams A and then Bt of every segment, and counts as one arrival on each operand's counter
+    a.single_producer = t.num_producer_waves == 1;
+    a.pa = a.single_producer ? 1 : t.num_producer_waves / 2;
+    a.pb = a.single_producer ? 1 : t.num_producer_waves - a.pa;
     a.bar_steps_a = mode == CK_SYNC_TILE ? 0 : t.bar_steps_a;
     a.bar_steps_b = mode == CK_SYNC_TILE ? 0 : t.bar_steps_b;
-    a.swizzle = g_swizzle.load();
-    a.num_xcd = g_num_xcd.load();
+    a.swizzle = opt[OPT_SWIZZLE];
+    a.num_xcd = opt[OPT_NUM_XCD];
     // one vector access per accumulator block: 16 bytes of fp32 need only the 4-byte alignment checked above
     // (any N); 8 bytes of 16-bit results need their own alignment
     a.vec_store = !out16 || ((N % 4 == 0) && !((uintptr_t)D & 7) && (beta == 0.f || !((uintptr_t)C & 7)));
     // Non-temporal stores of D pay where the stores of a row fill whole 128-byte lines; rows that start anywhere make
     // every 128-byte run straddle two lines, and only ordinary stores let the two parts meet in L2.
-    const int store_policy = g_d_store_policy.load();
+    const int store_policy = opt[OPT_D_STORE_POLICY];
     auto whole_lines = [](const void* base, int64_t row_bytes) { return (uintptr_t)base % LINE_BYTES == 0 && row_bytes % LINE_BYTES == 0; };
     a.nt_store = store_policy == 1 || (store_policy == 0 && whole_lines(D, (int64_t)N * (out16 ? 2 : 4)));
-    a.spin_limit = (uint32_t)g_spin_limit.load();
-    a.prio_mode = g_prio_mode.load();
-    a.producer_nap = g_producer_nap.load();
+    a.spin_limit = (uint32_t)opt[OPT_SPIN_LIMIT];
+    a.prio_mode = opt[OPT_PRIO_MODE];
+    a.producer_nap = opt[OPT_PRODUCER_NAP];
     const int src = status_ptr_for_current_device(&a.status);
     if (src != CK_OK) return src;
 
     const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
-    const int grid = persistent_grid(tiles, t.num_cus, a.num_xcd, g_even_rounds.load() != 0);
+    const int grid = persistent_grid(tiles, t.num_cus, a.num_xcd, opt[OPT_EVEN_ROUNDS] != 0);
     const dim3 block((t.num_producer_waves + t.num_consumer_waves) * WAVE);
     const size_t lds = (size_t)gemm_lds_bytes(t);
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e = hipErrorInvalidValue;
     a.split_k = 1;
     a.split_chunk = 32;
-    if (g_straight_line.load() &&
-        gemm_stream_applies(a, t.tile_dim, t.segment_dim_k, t.num_stages, t.num_producer_waves, t.num_consumer_waves)) {
-        // Tile width and K slices from the cost model: few tiles and a deep K are cut into slices so that every CU
-        // has an item (partial products into scratch memory, one reduction pass); tile counts that leave much of the
-        // device idle take 256 x 128 tiles.
-        const bool bek = g_barrier_every_kstep.load() != 0;
-        const StreamPlan plan = stream_plan(M, N, K, t.num_cus);
-        int slices = plan.slices;
+    a.whole_tiles = (int)tiles;
+    a.fix_partials = nullptr;
+    a.fix_state = nullptr;
+    if (straight_line_tuple(t, opt) && gemm_stream_applies(a, t.tile_dim, t.segment_dim_k, t.num_stages, t.num_producer_waves, t.num_consumer_waves)) {
+        // Tile width, K slices and grid from the cost model: few tiles and a deep K are cut into slices so that every CU
+        // has an item; the partly filled last round of many tiles likewise; tile counts that leave much of the device idle
+        // take 256 x 128 tiles.
+        const bool bek = opt[OPT_BARRIER_EVERY_KSTEP] != 0;
+        StreamPlan plan = stream_plan(M, N, K, t.num_cus, opt);
         const bool half = plan.half_width;
-        const int64_t stream_tiles = plan.tiles;   // tiles of the chosen width
         if (half) a.tiles_n = (N + 127) / 128;
-        const int stream_grid = persistent_grid(stream_tiles, t.num_cus, a.num_xcd, g_even_rounds.load() != 0);
         const long long count = (long long)M * N;
+        auto launch = [&](const GemmArgs& args, int wgs) {
+            return dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(wgs), s, args, bek, half) : launch_gemm_stream_bf16(dim3(wgs), s, args, bek, half);
+        };
+        // the K slices' scratch memory: a provided buffer that is too small is the caller's error; a failed allocation
+        // is not - the launch of whole tiles computes the same product without any
+        void* state = nullptr;
         float* ws = nullptr;
-        if (slices > 1) {
-            const int trc = scratch_take(sc, (size_t)slices * count * sizeof(float), s, (void**)&ws);
-            // a provided buffer that is too small is the caller's error; a failed allocation is not: the
-            // single-pass launch computes the same product without any
+        if (plan.slices > 1) {
+            int trc = CK_OK;
+            if (plan.fused) {
+                trc = scratch_take(sc, fix_state_bytes(plan), s, &state);
+                if (trc == CK_OK) {
+                    trc = scratch_take(sc, fix_partial_bytes(plan), s, (void**)&ws);
+                    if (trc != CK_OK) (void)scratch_release(sc, state, s);
+                }
+            } else {
+                trc = scratch_take(sc, (size_t)plan.slices * count * sizeof(float), s, (void**)&ws);
+            }
             if (trc == CK_ERR_TOO_LARGE) return trc;
-            if (trc != CK_OK) slices = 1;
+            if (trc != CK_OK) {
+                plan.slices = 1; plan.whole_tiles = plan.tiles; plan.fused = false;
+                plan.grid = persistent_grid(plan.tiles, t.num_cus, a.num_xcd, opt[OPT_EVEN_ROUNDS] != 0);
+            }
         }
-        if (slices == 1) {
-            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(stream_grid), s, a, bek, half) : launch_gemm_stream_bf16(dim3(stream_grid), s, a, bek, half);
+        const int64_t sliced_tiles = plan.tiles - plan.whole_tiles;
+        if (plan.slices == 1) {
+            e = launch(a, plan.grid);
+        } else if (plan.fused) {
+            // one launch: the whole tiles, then the (tile, slice) items; a wave tile's last slice to arrive adds the others
+            GemmArgs p = a;
+            p.split_k = plan.slices;
+            p.whole_tiles = (int)plan.whole_tiles;
+            // sliced items are dealt slice by slice in runs of split_chunk tiles: 32 (what an XCD runs at a time) when the
+            // sliced tiles come in whole runs of 32, otherwise all of them in one run
+            p.split_chunk = sliced_tiles % 32 == 0 ? 32 : (int)sliced_tiles;
+            p.fix_state = static_cast<unsigned int*>(state);
+            p.fix_partials = ws;
+            const long long words = (long long)(fix_state_bytes(plan) / 4);
+            hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)std::min<long long>((words + 255) / 256, 1024)), dim3(256), 0, s, p.fix_state, words);
+            e = hipGetLastError();
+            if (e == hipSuccess) e = launch(p, plan.grid);
+            if (!scratch_release(sc, ws, s) && e == hipSuccess) e = hipErrorUnknown;
+            if (!scratch_release(sc, state, s) && e == hipSuccess) e = hipErrorUnknown;
         } else {
             GemmArgs p = a;
-            p.split_k = slices;
-            // items are dealt slice by slice in runs of split_chunk tiles: 32 (what an XCD runs at a time) when the tiles
-            // come in whole runs of 32, otherwise all tiles of a slice in one run
-            p.split_chunk = stream_tiles % 32 == 0 ? 32 : (int)stream_tiles;
+            p.split_k = plan.slices;
+            p.whole_tiles = 0;
+            p.split_chunk = plan.tiles % 32 == 0 ? 32 : (int)plan.tiles;
             p.D = ws; p.C = nullptr; p.alpha = 1.f; p.beta = 0.f; p.out16 = 0; p.vec_store = 1;
             p.nt_store = store_policy == 1 || (store_policy == 0 && whole_lines(ws, (int64_t)N * 4) && count * 4 % LINE_BYTES == 0);
-            const int64_t items = stream_tiles * slices;
-            const int pgrid = (int)(items < t.num_cus ? items : t.num_cus);
-            e = dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(pgrid), s, p, bek, half) : launch_gemm_stream_bf16(dim3(pgrid), s, p, bek, half);
+            e = launch(p, plan.grid);
             if (e == hipSuccess) {
                 const unsigned blocks = (unsigned)((count + 255) / 256 < 65535 * 8 ? (count + 255) / 256 : 65535 * 8);
                 const bool vec4 = !out16 && count % 4 == 0 && ((uintptr_t)D | (uintptr_t)(beta != 0.f ? C : nullptr)) % 16 == 0;
+                const int slices = plan.slices;
                 if (vec4) {
                     const long long count4 = count / 4;
                     const unsigned b4 = (unsigned)((count4 + 255) / 256 < 65535 * 8 ? (count4 + 255) / 256 : 65535 * 8);
@@ -464,7 +614,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     } else if (t.num_producer_waves == 0) {
         e = dtype == CK_DT_F16 ? launch_gemm_fused_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a)
                                : launch_gemm_fused_bf16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), lds, s, a);
-    } else if (mode == CK_SYNC_TILE && t.num_stages >= 2 && g_tile_sync_barrier.load()) {
+    } else if (mode == CK_SYNC_TILE && t.num_stages >= 2 && opt[OPT_TILE_SYNC_BARRIER] && !a.single_producer && t.segment_dim_k <= 128) {
         // tile granularity through the workgroup barrier: the ring is the whole LDS allocation
         const size_t ring = (size_t)t.num_stages * 2 * stage_bytes_one_operand(t.tile_dim, t.segment_dim_k);
         e = dtype == CK_DT_F16 ? launch_gemm_pcb_f16(t.tile_dim, t.segment_dim_k, t.num_consumer_waves, dim3(grid), block, ring, s, a)
@@ -486,90 +636,106 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
 
 extern "C" {
 
-int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* Bt, const float* C, float* D,
-                                         float alpha, float beta, int M, int N, int K, int tile_dim,
-                                         int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
-                                         int bar_step_rows_b, int tile_group_m, int num_stages,
-                                         int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
-    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0, Scratch{Scratch::ALLOCATE, nullptr, 0});
+#define CK_TUNING_PARAMS int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, \
+                         int tile_group_m, int num_stages, int num_producer_waves, int num_consumer_waves, int num_cus
+#define CK_TUNING_VALUE ck::GemmTuning{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, tile_group_m, \
+                                       num_stages, num_producer_waves, num_consumer_waves, num_cus, 0}
+
+int ckopt_launch_options_init(ckopt_launch_options* options) {
+    if (!options) return ck::CK_ERR_NULL;
+    const Options o = default_options();
+    options->struct_bytes = (int)sizeof(ckopt_launch_options);
+    int* f = &options->lds_swizzle;
+    for (int k = 0; k < NUM_OPTIONS; ++k) f[k] = o.v[k];
+    return ck::CK_OK;
 }
 
-int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void* Bt, const void* C, void* D,
-                                            float alpha, float beta, int M, int N, int K, int tile_dim,
-                                            int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
-                                            int bar_step_rows_b, int tile_group_m, int num_stages,
-                                            int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
-    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 1, Scratch{Scratch::ALLOCATE, nullptr, 0});
+int ckopt_gemm_shmem_tc_async_opt_port_2(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta,
+                                         int M, int N, int K, CK_TUNING_PARAMS, void* stream) {
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, CK_TUNING_VALUE, default_options(), stream, 0, Scratch{Scratch::ALLOCATE, nullptr, 0});
 }
 
-int ckopt_gemm_shmem_tc_async_opt_port_2_noalloc(int dtype, const void* A, const void* Bt, const float* C, float* D,
-                                                 float alpha, float beta, int M, int N, int K, int tile_dim,
-                                                 int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
-                                                 int bar_step_rows_b, int tile_group_m, int num_stages,
-                                                 int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
-    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+int ckopt_gemm_shmem_tc_async_opt_port_2_lp(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta,
+                                            int M, int N, int K, CK_TUNING_PARAMS, void* stream) {
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, CK_TUNING_VALUE, default_options(), stream, 1, Scratch{Scratch::ALLOCATE, nullptr, 0});
+}
+
+int ckopt_gemm_shmem_tc_async_opt_port_2_noalloc(int dtype, const void* A, const void* Bt, const float* C, float* D, float alpha, float beta,
+                                                 int M, int N, int K, CK_TUNING_PARAMS, void* stream) {
     unsigned char* ptr = nullptr;
     const int rc = static_scratch_for_current_device(&ptr);
     if (rc != ck::CK_OK) return rc;
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0,
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, CK_TUNING_VALUE, default_options(), stream, 0,
                        Scratch{Scratch::PROVIDED, reinterpret_cast<char*>(ptr), (size_t)CKOPT_NOALLOC_SCRATCH_BYTES});
 }
 
-int64_t ckopt_gemm_workspace_bytes(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a,
-                                   int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
-                                   int num_producer_waves, int num_consumer_waves, int num_cus) {
-    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+int ckopt_gemm_shmem_tc_async_opt_port_2_ex(int dtype, int cd_dtype, const void* A, const void* Bt, const void* C, void* D, float alpha,
+                                            float beta, int M, int N, int K, CK_TUNING_PARAMS, const ckopt_launch_options* options,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+    Options opt;
+    const int orc = options_from_public(options, &opt);
+    if (orc != ck::CK_OK) return orc;
+    if (!(cd_dtype == ck::CK_DT_F32 || cd_dtype == dtype)) return ck::CK_ERR_BAD_PARAM;
+    const Scratch sc = workspace ? Scratch{Scratch::PROVIDED, static_cast<char*>(workspace), workspace_bytes} : Scratch{Scratch::ALLOCATE, nullptr, 0};
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, CK_TUNING_VALUE, opt, stream, cd_dtype == ck::CK_DT_F32 ? 0 : 1, sc);
+}
+
+int64_t ckopt_gemm_workspace_bytes_ex(int M, int N, int K, int operands_aligned, CK_TUNING_PARAMS, const ckopt_launch_options* options) {
+    Options opt;
+    const int orc = options_from_public(options, &opt);
+    if (orc != ck::CK_OK) return orc;
+    const ck::GemmTuning t = CK_TUNING_VALUE;
     if (M <= 0 || N <= 0 || K <= 0) return ck::CK_ERR_BAD_PARAM;
     const int rc = ck::check_gemm_tuning(t);
     if (rc != ck::CK_OK) return rc;
-    const size_t need = scratch_need(M, N, K, operands_aligned != 0, t);
+    const size_t need = scratch_need(M, N, K, operands_aligned != 0, t, opt);
     return need ? (int64_t)(need + SCRATCH_ALIGN) : 0;  // room to start on a 256-byte boundary inside any buffer
 }
+int64_t ckopt_gemm_workspace_bytes(int M, int N, int K, int operands_aligned, CK_TUNING_PARAMS) {
+    return ckopt_gemm_workspace_bytes_ex(M, N, K, operands_aligned, tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
+                                         bar_step_rows_b, tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus, nullptr);
+}
 
-int ckopt_gemm_launch_plan(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b,
-                           int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages, int num_producer_waves,
-                           int num_consumer_waves, int num_cus, int* plan_out) {
-    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+int ckopt_gemm_launch_plan_ex(int M, int N, int K, int operands_aligned, CK_TUNING_PARAMS, const ckopt_launch_options* options, int* plan_out) {
+    Options opt;
+    const int orc = options_from_public(options, &opt);
+    if (orc != ck::CK_OK) return orc;
+    const ck::GemmTuning t = CK_TUNING_VALUE;
     if (!plan_out) return ck::CK_ERR_NULL;
     if (M <= 0 || N <= 0 || K <= 0) return ck::CK_ERR_BAD_PARAM;
     const int rc = ck::check_gemm_tuning(t);
     if (rc != ck::CK_OK) return rc;
-    const bool copies = K % ck::CHUNK_ELEMS != 0 || !operands_aligned;
-    const int k = copies ? padded_k(K, t) : K;
+    const bool copies = needs_copies(K, operands_aligned != 0);
     plan_out[0] = 0; plan_out[1] = t.tile_dim; plan_out[2] = 1; plan_out[3] = copies ? 1 : 0;
-    if (straight_line_tuple(t)) {
-        const StreamPlan plan = stream_plan(M, N, k, t.num_cus);
+    plan_out[4] = 0; plan_out[5] = 0; plan_out[6] = 0;
+    if (straight_line_tuple(t, opt)) {
+        const StreamPlan plan = stream_plan(M, N, launch_k(K, operands_aligned != 0, t, opt), t.num_cus, opt);
         plan_out[0] = 1;
         plan_out[1] = plan.half_width ? 128 : 256;
         plan_out[2] = plan.slices;
+        plan_out[4] = (int)(plan.tiles - plan.whole_tiles);
+        plan_out[5] = plan.slices > 1 && plan.fused ? 1 : 0;
+        plan_out[6] = plan.grid;
     }
     return ck::CK_OK;
 }
+int ckopt_gemm_launch_plan(int M, int N, int K, int operands_aligned, CK_TUNING_PARAMS, int* plan_out) {
+    return ckopt_gemm_launch_plan_ex(M, N, K, operands_aligned, tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a,
+                                     bar_step_rows_b, tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus, nullptr, plan_out);
+}
 
-int ckopt_gemm_shmem_tc_async_opt_port_2_ws(int dtype, int cd_dtype, const void* A, const void* Bt, const void* C, void* D,
-                                            float alpha, float beta, int M, int N, int K, int tile_dim, int segment_dim_k,
-                                            int bar_steps_a, int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b,
-                                            int tile_group_m, int num_stages, int num_producer_waves, int num_consumer_waves,
-                                            int num_cus, void* workspace, size_t workspace_bytes, void* stream) {
-    const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+int ckopt_gemm_shmem_tc_async_opt_port_2_ws(int dtype, int cd_dtype, const void* A, const void* Bt, const void* C, void* D, float alpha,
+                                            float beta, int M, int N, int K, CK_TUNING_PARAMS, void* workspace, size_t workspace_bytes,
+                                            void* stream) {
     if (!(cd_dtype == ck::CK_DT_F32 || cd_dtype == dtype)) return ck::CK_ERR_BAD_PARAM;
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, cd_dtype == ck::CK_DT_F32 ? 0 : 1,
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, CK_TUNING_VALUE, default_options(), stream, cd_dtype == ck::CK_DT_F32 ? 0 : 1,
                        Scratch{Scratch::PROVIDED, static_cast<char*>(workspace), workspace ? workspace_bytes : 0});
 }
 
-int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
-                                         float alpha, float beta, int M, int N, int K, int tile_dim,
-                                         int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
-                                         int tile_group_m, int num_stages, int num_producer_waves,
-                                         int num_consumer_waves, int num_cus, void* stream) {
+// port_1: every wave tile (or every 16-row block) has its own signal = port_2 with maximal bar_steps
+static int launch_port_1(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M, int N, int K,
+                         int tile_dim, int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
+                         int num_producer_waves, int num_consumer_waves, int num_cus, void* stream, int out16) {
     if (!(num_consumer_waves == 4 || num_consumer_waves == 8) || !(tile_dim == 64 || tile_dim == 128 || tile_dim == 256))
         return ck::CK_ERR_BAD_PARAM;
     const int mode = ck::sync_mode_of(tile_dim, num_consumer_waves, bar_step_rows_a, bar_step_rows_b);
@@ -580,17 +746,47 @@ int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* B
         sb = ck::wave_tile_cols(tile_dim, num_consumer_waves) - 1;
     }
     const ck::GemmTuning t{tile_dim, segment_dim_k, sa, sb, bar_step_rows_a, bar_step_rows_b,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0, Scratch{Scratch::ALLOCATE, nullptr, 0});
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus, 0};
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, default_options(), stream, out16, Scratch{Scratch::ALLOCATE, nullptr, 0});
+}
+int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
+                                         float alpha, float beta, int M, int N, int K, int tile_dim,
+                                         int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
+                                         int tile_group_m, int num_stages, int num_producer_waves,
+                                         int num_consumer_waves, int num_cus, void* stream) {
+    return launch_port_1(dtype, A, Bt, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_step_rows_a, bar_step_rows_b, tile_group_m,
+                         num_stages, num_producer_waves, num_consumer_waves, num_cus, stream, 0);
+}
+int ckopt_gemm_shmem_tc_async_opt_port_1_lp(int dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim,
+                                            int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
+                                            int tile_group_m, int num_stages, int num_producer_waves,
+                                            int num_consumer_waves, int num_cus, void* stream) {
+    return launch_port_1(dtype, A, Bt, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, bar_step_rows_a, bar_step_rows_b, tile_group_m,
+                         num_stages, num_producer_waves, num_consumer_waves, num_cus, stream, 1);
 }
 
+// port_0: one signal pair per stage; its legal set also holds a single producer wave (port_0.cu:538)
+static int launch_port_0(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M, int N, int K,
+                         int tile_dim, int segment_dim_k, int tile_group_m, int num_stages, int num_producer_waves, int num_consumer_waves,
+                         int num_cus, void* stream, int out16) {
+    const ck::GemmTuning t{tile_dim, segment_dim_k, 0, 0, tile_dim, tile_dim, tile_group_m, num_stages, num_producer_waves, num_consumer_waves,
+                           num_cus, 1};
+    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, default_options(), stream, out16, Scratch{Scratch::ALLOCATE, nullptr, 0});
+}
 int ckopt_gemm_shmem_tc_async_opt_port_0(int dtype, const void* A, const void* Bt, const float* C, float* D,
                                          float alpha, float beta, int M, int N, int K, int tile_dim,
                                          int segment_dim_k, int tile_group_m, int num_stages,
                                          int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
-    const ck::GemmTuning t{tile_dim, segment_dim_k, 0, 0, tile_dim, tile_dim,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
-    return gemm_launch(dtype, A, Bt, C, D, alpha, beta, M, N, K, t, stream, 0, Scratch{Scratch::ALLOCATE, nullptr, 0});
+    return launch_port_0(dtype, A, Bt, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, tile_group_m, num_stages, num_producer_waves,
+                         num_consumer_waves, num_cus, stream, 0);
+}
+int ckopt_gemm_shmem_tc_async_opt_port_0_lp(int dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim,
+                                            int segment_dim_k, int tile_group_m, int num_stages,
+                                            int num_producer_waves, int num_consumer_waves, int num_cus, void* stream) {
+    return launch_port_0(dtype, A, Bt, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k, tile_group_m, num_stages, num_producer_waves,
+                         num_consumer_waves, num_cus, stream, 1);
 }
 
 int ckopt_get_lds_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
@@ -624,7 +820,7 @@ int ckopt_check_gemm_tuning(int tile_dim, int segment_dim_k, int bar_steps_a, in
                             int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
                             int num_producer_waves, int num_consumer_waves, int num_cus) {
     const ck::GemmTuning t{tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
-                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus};
+                           tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus, 0};
     return ck::check_gemm_tuning(t);
 }
 
@@ -632,8 +828,8 @@ int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out)
     using namespace ck;
     if (!tuning_out) return CK_ERR_NULL;
     if (M <= 0 || N <= 0 || K <= 0 || num_cus <= 0) return CK_ERR_BAD_PARAM;
+    const Options opt = default_options();
     auto tiles = [&](int t) { return (int64_t)((M + t - 1) / t) * ((N + t - 1) / t); };
-    const int kp = (K + STREAM_K_MULTIPLE_HOST - 1) / STREAM_K_MULTIPLE_HOST * STREAM_K_MULTIPLE_HOST;  // K of the straight-line tuple after the repack
     // {tile, seg_k, bar_steps_a, bar_steps_b, rows_a, rows_b, group, stages, producers, consumers}
     static const int straight_line[10] = {256, 32, 0, 0, 256, 256, 4, 5, 0, 8};
     static const int fused_128[10] = {128, 128, 0, 0, 128, 128, 4, 2, 0, 8};
@@ -641,16 +837,18 @@ int ckopt_suggest_gemm_tuning(int M, int N, int K, int num_cus, int* tuning_out)
     static const int pc_256[10] = {256, 64, 0, 0, 256, 256, 4, 2, 2, 8};
     const int* pick = fused_64;
     const int64_t t256 = tiles(256);
-    const bool straight_ok = g_straight_line.load() && g_swizzle.load();
+    const bool straight_ok = opt[OPT_STRAIGHT_LINE] && opt[OPT_SWIZZLE];
     if (!straight_ok) {
         // without the straight-line kernel: the reference's design on 256 tiles when they fill half the device
         if (t256 * 2 >= num_cus) pick = pc_256;
         else if (tiles(128) * 2 >= num_cus) pick = fused_128;
     } else {
-        // the shortest of three estimates: the straight-line kernel with the tile width and slice count the launcher
-        // would choose (stream_plan), and the general kernel on 128 and on 64 tiles - one workgroup per CU, measured per
-        // 128 of K: 1.4 us for a 128 x 128 tile, 0.65 us for a 64 x 64 tile, about 4 us per round besides
-        const double straight_us = stream_plan(M, N, kp, num_cus).us;
+        // the shortest of three estimates: the straight-line kernel as the launcher would run it on aligned operands (its K,
+        // tile width and slice count: launch_k, stream_plan), and the general kernel on 128 and on 64 tiles - one
+        // workgroup per CU, measured per 128 of K: 1.4 us for a 128 x 128 tile, 0.65 us for a 64 x 64 tile, about 4 us
+        // per round besides
+        const GemmTuning st{256, 32, 0, 0, 256, 256, 4, 5, 0, 8, num_cus, 0};
+        const double straight_us = stream_plan(M, N, launch_k(K, true, st, opt), num_cus, opt).us;
         auto general_us = [&](int t, double seg_us) { return std::ceil((double)tiles(t) / num_cus) * ((double)K / 128.0 * seg_us + 4.0); };
         const double us_128 = general_us(128, 1.4), us_64 = general_us(64, 0.65);
         if (straight_us <= us_128 && straight_us <= us_64) pick = straight_line;
@@ -719,21 +917,10 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
 }
 
 int ckopt_set_option(int key, int value) {
-    switch (key) {
-        case 0: return g_swizzle.exchange(value != 0);
-        case 1: if (value < 1) return ck::CK_ERR_BAD_PARAM; return g_spin_limit.exchange(value);
-        case 2: if (value < 1 || value > 64) return ck::CK_ERR_BAD_PARAM; return g_num_xcd.exchange(value);
-        case 3: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_prio_mode.exchange(value);
-        case 4: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_producer_nap.exchange(value);
-        case 5: return g_tile_sync_barrier.exchange(value != 0);
-        case 6: return g_straight_line.exchange(value != 0);
-        case 7: if (value < 0 || value > 16) return ck::CK_ERR_BAD_PARAM; return g_split_k.exchange(value);
-        case 8: return g_barrier_every_kstep.exchange(value != 0);
-        case 9: return g_even_rounds.exchange(value != 0);
-        case 10: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_d_store_policy.exchange(value);
-        case 11: if (value < 0 || value > 2) return ck::CK_ERR_BAD_PARAM; return g_half_width.exchange(value);
-        default: return ck::CK_ERR_BAD_PARAM;
-    }
+    if (key < 0 || key >= NUM_OPTIONS) return ck::CK_ERR_BAD_PARAM;
+    if (OPTION_RULES[key].hi == 1) value = value != 0;   // switches take any non-zero value as on
+    if (value < OPTION_RULES[key].lo || value > OPTION_RULES[key].hi) return ck::CK_ERR_BAD_PARAM;
+    return g_option[key].exchange(value);
 }
 
 const char* ckopt_error_string(int code) {

@@ -105,7 +105,8 @@ CK_HD int chunks_per_row(int segment_dim_k) { return segment_dim_k / CHUNK_ELEMS
 CK_HD int swizzle_key(int row, int cpr) {
     // Found conflict-free for ds_read_b128 on gfx950 by measurement (64 banks, 256 B/clk): rows of
     // 64 and 128 bytes rotate with every second row, rows of 256 bytes with every row.
-    return cpr == 16 ? row % 16 : (row >> 1) % cpr;
+    // (rows of 512 bytes: as rows of 256 - the key moves a chunk inside its 256-byte half)
+    return cpr >= 16 ? row % 16 : (row >> 1) % cpr;
 }
 // slot (physical chunk index inside the row) that holds logical chunk c of row `row`
 CK_HD int swizzle_slot(int row, int c, int cpr, int swizzle_on) { return swizzle_on ? (c ^ swizzle_key(row, cpr)) : c; }
@@ -155,6 +156,7 @@ CK_HD int get_lds_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_
 struct GemmTuning {
     int tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b;
     int tile_group_m, num_stages, num_producer_waves, num_consumer_waves, num_cus;
+    int port_0_rules;  // the legal set of the port_0 launcher: also one producer wave (port_0.cu:538)
 };
 
 // Largest total wave count (producers + consumers) a kernel instance is compiled for. It fixes the
@@ -170,10 +172,12 @@ CK_HD int gemm_lds_bytes(const GemmTuning& t) {
 
 CK_HD int check_gemm_tuning(const GemmTuning& t) {
     if (!(t.tile_dim == 64 || t.tile_dim == 128 || t.tile_dim == 256)) return CK_ERR_BAD_PARAM;
-    if (!(t.segment_dim_k == 32 || t.segment_dim_k == 64 || t.segment_dim_k == 128)) return CK_ERR_BAD_PARAM;
+    // the reference takes every multiple of 64 (port_2.cu:1113; port_0: of tile_dim / 2, port_0.cu:534); one MFMA eats 32 of K
+    if (t.segment_dim_k < MFMA_K || t.segment_dim_k % MFMA_K != 0) return CK_ERR_BAD_PARAM;
     if (!(t.num_consumer_waves == 4 || t.num_consumer_waves == 8)) return CK_ERR_BAD_PARAM;
-    // 0 producer waves: every consumer wave also streams its share of the segments (fused variant)
-    if (!(t.num_producer_waves == 0 || t.num_producer_waves == 2 || t.num_producer_waves == 4 || t.num_producer_waves == 8))
+    // 0 producer waves: every consumer wave also streams its share of the segments (fused variant); 1: port_0 only
+    if (!(t.num_producer_waves == 0 || t.num_producer_waves == 2 || t.num_producer_waves == 4 || t.num_producer_waves == 8 ||
+          (t.num_producer_waves == 1 && t.port_0_rules)))
         return CK_ERR_BAD_PARAM;
     if (t.num_stages < 1 || t.num_stages > MAX_STAGES) return CK_ERR_BAD_PARAM;
     if (t.tile_group_m < 1 || t.num_cus < 1) return CK_ERR_BAD_PARAM;
@@ -194,8 +198,12 @@ CK_HD int check_gemm_tuning(const GemmTuning& t) {
     // 64 accumulator blocks (256 registers) leave no room for a second wave on the SIMD
     if (get_num_acc(t.tile_dim, t.num_consumer_waves) > 32) return CK_ERR_NO_INSTANCE;
     if (t.num_producer_waves + t.num_consumer_waves > max_waves_for(t.tile_dim, t.num_consumer_waves)) return CK_ERR_NO_INSTANCE;
-    const int lds = gemm_lds_bytes(t);
+    const int64_t lds = t.segment_dim_k > 4096 ? (int64_t)LDS_BYTES_PER_CU + 1 : (int64_t)gemm_lds_bytes(t);
     if (lds > LDS_BYTES_PER_CU) return CK_ERR_LDS_BUDGET;
+    // kernel instances: 32, 64 and 128 deep segments everywhere; 256 deep ones in the producer/consumer kernel on 64 and
+    // 128 tiles (the depths the reference's drivers sweep, port_2.cu:1520-1564); every other legal depth has none
+    const bool deep = t.segment_dim_k == 256 && t.num_producer_waves > 0 && t.tile_dim <= 128;
+    if (!(t.segment_dim_k == 32 || t.segment_dim_k == 64 || t.segment_dim_k == 128 || deep)) return CK_ERR_NO_INSTANCE;
     return CK_OK;
 }
 

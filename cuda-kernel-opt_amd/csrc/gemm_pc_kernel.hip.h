@@ -57,7 +57,8 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     int nseg;  // ceil(K / segment_dim_k)
     int tile_group_m, num_stages;
-    int pa, pb;  // producer waves on A and on Bt
+    int pa, pb;  // producer waves on A and on Bt (arrivals per fill on each operand's "full" counters)
+    int single_producer;  // one producer wave streams A and then Bt of every segment (port_0's single producer warp); pa = pb = 1
     int bar_steps_a, bar_steps_b;
     int swizzle;
     int num_xcd;
@@ -65,9 +66,19 @@ struct GemmArgs {
     int out16;      // C and D hold the operands' 16-bit element type instead of fp32 (accumulation stays fp32)
     int nt_store;   // D's rows start on 128-byte lines: vector stores of D are non-temporal (they fill whole lines and need not
                     // stay in L2); otherwise ordinary stores, so that the two parts of a line written by different stores meet in L2
-    int split_k;    // straight-line kernel only: K is cut into this many slices (>= 1), one work item per (tile, slice);
-                    // slice s writes its partial products to D + s * M * N (a workspace; alpha 1, beta 0, fp32)
-    int split_chunk;  // consecutive work items that belong to one slice (32 = one XCD round, or all tiles if fewer)
+    int split_k;    // straight-line kernel only: the tiles from whole_tiles on are cut into this many K slices (>= 1), one
+                    // work item per (tile, slice). Without fix_partials slice s writes its partial products to
+                    // D + s * M * N (a workspace; alpha 1, beta 0, fp32) and a second kernel adds the planes.
+    int split_chunk;  // consecutive work items that belong to one slice (32 = one XCD round, or all sliced tiles if fewer)
+    int whole_tiles;  // straight-line kernel only: tile counts [0, whole_tiles) are work items over all of K; the K-sliced
+                      // items follow them in the item list (all tiles when split_k is 1)
+    // Reduction of the K slices inside the kernel (straight-line kernel): of a wave tile's accumulator block rows the
+    // wave of slice s keeps the rows i with i % split_k == s and stores the others to fix_partials; when all split_k
+    // waves have done so, each adds what the others stored for its rows and writes those rows of D. fix_state holds one
+    // word per (sliced tile, wave) that starts at zero: the number of waves that have stored. Null: no reduction in the
+    // kernel.
+    float* fix_partials;
+    unsigned int* fix_state;
     uint32_t spin_limit;
     int prio_mode;      // 0: producers at raised priority; 1: also asymmetric consumer burst priorities per SIMD pair; 2: none
     int producer_nap;   // s_sleep argument class of the producers' flag polling: 0 -> 1, 1 -> 4, 2 -> 16
@@ -75,7 +86,7 @@ struct GemmArgs {
                            // ticks workgroup 0 spent in the last launch (actual-clock evidence)
 };
 
-enum : unsigned { CK_STATUS_PRODUCER_TIMEOUT = 1u, CK_STATUS_CONSUMER_TIMEOUT = 2u };
+enum : unsigned { CK_STATUS_PRODUCER_TIMEOUT = 1u, CK_STATUS_CONSUMER_TIMEOUT = 2u, CK_STATUS_REDUCTION_TIMEOUT = 4u };
 
 struct f16_tag {};
 struct bf16_tag {};
@@ -329,7 +340,7 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
     constexpr int BLK_ROWS = MODE == CK_SYNC_TILE ? TILE : MODE == CK_SYNC_WAVE ? (IS_A ? WTR : WTC) * 16 : 16;
     constexpr int NBLK = TILE / BLK_ROWS;
     constexpr int NIB = BLK_ROWS / RPI;          // wave loads per row block
-    constexpr int VAR = CPR == 4 ? 1 : CPR == 8 ? 2 : 4;  // period of the swizzle key in E
+    constexpr int VAR = CPR == 4 ? 1 : CPR == 8 ? 2 : CPR == 16 ? 4 : 8;  // period of the swizzle key in E
     static_assert(BLK_ROWS % RPI == 0, "row block must be whole wave loads");
 
     const int sa = g.bar_steps_a, sb = g.bar_steps_b;
@@ -442,6 +453,75 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
                     if (sub < s_own) sq.push(fl + (full_off + unit * (s_own + 1) + sub) * 4);
                     else if (sub == WT - 1) sq.push(fl + (full_off + unit * (s_own + 1) + s_own) * 4);
                 }
+            }
+            if (++stage == S) { stage = 0; ++fill; }
+        }
+    }
+    sq.drain();
+}
+
+// The single producer wave of the port_0 launcher (port_0.cu:106-147 with one producer warp): tile granularity, the one
+// wave streams the A rows and then the Bt rows of every segment and is the one arrival on each operand's "full" counter.
+template <int TILE, int SEGK, int CW>
+__device__ __forceinline__ void produce_both(const GemmArgs& g, uint32_t flags_base, uint32_t ring_base, int lane) {
+    constexpr int CPR = SEGK / CHUNK_ELEMS, RB = SEGK * 2, RPI = WAVE / CPR, OPB = TILE * RB;
+    constexpr int NI = TILE / RPI;               // wave loads per operand stage
+    constexpr int VAR = CPR == 4 ? 1 : CPR == 8 ? 2 : CPR == 16 ? 4 : 8;
+    constexpr int FPS = 4;                        // counters per stage: full A, empty A, full Bt, empty Bt
+    const int S = g.num_stages;
+    const int64_t pitch = (int64_t)g.K * 2;
+    const uint32_t pitch32 = (uint32_t)pitch;
+    const int lane_row = lane / CPR, lane_slot = lane % CPR;
+    uint32_t lane_off[VAR];
+    int lane_chunk[VAR];
+#pragma unroll
+    for (int v = 0; v < VAR; ++v) {
+        lane_chunk[v] = swizzle_slot(v * RPI + lane_row, lane_slot, CPR, g.swizzle);
+        lane_off[v] = (uint32_t)lane_row * pitch32 + (uint32_t)lane_chunk[v] * CHUNK_BYTES;
+    }
+    const uint32_t load_step = (uint32_t)RPI * pitch32;
+    const int grid = gridDim.x;
+    const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
+    const int64_t total_tiles = (int64_t)g.tiles_m * g.tiles_n;
+    Spin sp{g.spin_limit, g.status, CK_STATUS_PRODUCER_TIMEOUT, false};
+    SignalQueue<3> sq;
+    sq.init();
+    int stage = 0;
+    uint32_t fill = 0;
+    for (int64_t tc = slot; tc < total_tiles; tc += grid) {
+        const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
+        for (int seg = 0; seg < g.nseg; ++seg) {
+            stage = __builtin_amdgcn_readfirstlane(stage);
+            fill = __builtin_amdgcn_readfirstlane(fill);
+            const uint32_t fl = flags_base + (uint32_t)stage * FPS * 4;
+            const int k0 = seg * SEGK;
+#pragma unroll
+            for (int op = 0; op < 2; ++op) {
+                const int row0 = __builtin_amdgcn_readfirstlane((op == 0 ? rc.row : rc.col) * TILE);
+                int rows_here = (op == 0 ? g.M : g.N) - row0;
+                rows_here = rows_here < TILE ? rows_here : TILE;
+                const uint32_t num_records = (uint32_t)((int64_t)rows_here * pitch);
+                __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                    (void*)((const char*)(op == 0 ? g.A : g.Bt) + (int64_t)row0 * pitch), 0, (int)num_records, 0x00020000);
+                const uint32_t st_base = ring_base + (uint32_t)stage * (2 * OPB) + (op == 0 ? 0 : OPB);
+                producer_wait(fl + (op == 0 ? 1 : 3) * 4, CW * fill, sq, sp, g.producer_nap);
+                if (rows_here == TILE && k0 + SEGK <= g.K) {
+#pragma unroll
+                    for (int E = 0; E < NI; ++E) {
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (CK_LDS void*)(uintptr_t)(st_base + (uint32_t)E * 1024u), 16,
+                                                                 lane_off[E % VAR], (uint32_t)k0 * 2u + (uint32_t)E * load_step, 0, 0);
+                        sq.issued++;
+                    }
+                } else {
+#pragma unroll
+                    for (int E = 0; E < NI; ++E) {
+                        uint32_t voff = lane_off[E % VAR] + (uint32_t)E * load_step + (uint32_t)k0 * 2u;
+                        if (k0 + lane_chunk[E % VAR] * CHUNK_ELEMS >= g.K) voff = num_records;  // absent k: zero fill
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (CK_LDS void*)(uintptr_t)(st_base + (uint32_t)E * 1024u), 16, voff, 0, 0, 0);
+                        sq.issued++;
+                    }
+                }
+                sq.push(fl + (op == 0 ? 0 : 2) * 4);
             }
             if (++stage == S) { stage = 0; ++fill; }
         }
@@ -651,6 +731,22 @@ __global__ __launch_bounds__(MAXW * 64) void gemm_pc_kernel(const GemmArgs g) {
 
     const uint32_t flags_base = lds0, ring_base = lds0 + fregion;
     // producers are rarely runnable and must issue their loads promptly when they are
+    if (MODE == CK_SYNC_TILE && g.single_producer) {
+        if constexpr (MODE == CK_SYNC_TILE) {
+            if (wave == 0) {
+                if (g.prio_mode != 2) __builtin_amdgcn_s_setprio(3);
+                produce_both<TILE, SEGK, CW>(g, flags_base, ring_base, lane);
+            } else if (wave < 1 + CW) {
+                consume<DT, TILE, SEGK, CW, MODE>(g, flags_base, ring_base, wave - 1, lane);
+                if (blockIdx.x == 0 && threadIdx.x == blockDim.x - 1) {
+                    const unsigned long long dc = clock64() - clk0, dw = wall_clock64() - wall0;
+                    g.status[2] = (unsigned)dc; g.status[3] = (unsigned)(dc >> 32);
+                    g.status[4] = (unsigned)dw; g.status[5] = (unsigned)(dw >> 32);
+                }
+            }
+        }
+        return;
+    }
     if (wave < g.pa + g.pb && g.prio_mode != 2) __builtin_amdgcn_s_setprio(3);
     if (wave < g.pa) {
         produce_px<TILE, SEGK, CW, MODE, true>(g, flags_base, ring_base, wave, g.pa, lane);

@@ -51,6 +51,7 @@ constexpr int STREAM_TILE_N_HALF = 128;   // the half-width form: 256 x 128 tile
 // bytes of the ring for tiles of 256 x tile_n
 constexpr int stream_lds_bytes(int tile_n) { return STREAM_STAGES * (STREAM_TILE + tile_n) * STREAM_SEGK * 2; }
 constexpr int STREAM_LDS_BYTES = stream_lds_bytes(STREAM_TILE);
+constexpr int FIX_STATE_STRIDE_BYTES = 128;  // bytes between the announcement counters of two (sliced tile, wave) units
 
 // KTAIL: K is a multiple of 8 but not of 64. The last loop body of a tile then reaches past K: its loads take
 // per-lane offsets in which every 16-byte chunk at or beyond K lies outside the descriptor (reads as zeros), chosen
@@ -87,6 +88,10 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     constexpr int FPC = (WTR + WTC + (WTC - PRE) - 1) / (WTC - PRE);   // fragments of the next k-step fetched per column
     static_assert(PRE >= 1 && (WTC - PRE) * FPC >= WTR + WTC && LOAD_COL_0 >= PRE && LOAD_COL_1 > LOAD_COL_0 && LOAD_COL_1 < WTC, "schedule");
     static_assert(LPB + EPILOGUE_STORES < 64 && EPILOGUE_STORES_16 < EPILOGUE_STORES, "the wait immediates must fit the 6-bit counter");
+    // 16-bit output whose rows are off the 16-byte boundaries (d16_misaligned) goes through the per-block epilogue, one
+    // store per accumulator block, while the landing wait behind it counts EPILOGUE_STORES: an epilogue that issues fewer
+    // stores than the wait counts would let fragments be read before their loads have landed
+    static_assert(WTR * WTC >= EPILOGUE_STORES, "the per-block epilogue issues at least the stores the landing wait counts");
     static_assert(NQ * QB == stream_lds_bytes(TILE_N) && NQ * QB <= LDS_BYTES_PER_CU, "the ring (all of the LDS for 256 x 256 tiles)");
 
     extern __shared__ __attribute__((aligned(1024))) char ck_smem[];
@@ -97,21 +102,30 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 
     const int grid = gridDim.x;
     const int slot = xcd_slot(blockIdx.x, grid, g.num_xcd);
-    // Work items: one per (tile, K slice). Item numbers are dealt like tile counts (slot, slot + grid, ...);
-    // 32 consecutive items - what one XCD runs at a time - are 32 consecutive tile counts of ONE slice
-    // (all tiles, if there are fewer than 32), so they share operand panels in that XCD's L2 exactly as
-    // whole tiles do. Without split-K an item is a tile count.
+    // Work items, dealt like tile counts (slot, slot + grid, ...): first the tile counts [0, T1) over all of K, then one
+    // item per (tile, K slice) for the tile counts from T1 on - the partly filled last round of a large launch, or every
+    // tile of a launch with fewer tiles than CUs. 32 consecutive sliced items - what one XCD runs at a time - are 32
+    // consecutive tile counts of ONE slice (all sliced tiles, if they do not come in whole runs of 32), so they share
+    // operand panels in that XCD's L2 exactly as whole tiles do. Without split-K every item is a tile count.
     const int S = g.split_k;
-    const int total_items = g.tiles_m * g.tiles_n * S;
+    const int T = g.tiles_m * g.tiles_n;
+    const int T1 = S > 1 ? g.whole_tiles : T;
+    const int total_items = T1 + (T - T1) * S;
     const int my_tiles = slot < total_items ? (total_items - slot + grid - 1) / grid : 0;
     const int kslice = g.K / S;                  // the host makes this a multiple of one loop body (KTAIL: S is 1, of 8)
-    const uint32_t kslice_bytes = (uint32_t)kslice * 2u;
-    const int nb = (kslice + STREAM_K_MULTIPLE - 1) / STREAM_K_MULTIPLE;   // loop bodies per item
+    const uint32_t kslice_bytes = (uint32_t)kslice * 2u, kwhole_bytes = (uint32_t)g.K * 2u;
+    const int nb_slice = (kslice + STREAM_K_MULTIPLE - 1) / STREAM_K_MULTIPLE;   // loop bodies per sliced item
+    const int nb_whole = (g.K + STREAM_K_MULTIPLE - 1) / STREAM_K_MULTIPLE;      // and per whole tile
     const int CH = g.split_chunk;
+    // tile count of an item; slice: its K slice, or -1 for a whole tile
     auto item_tile = [&](int64_t item, int& slice) __attribute__((always_inline)) {
-        const int64_t chunk = item / CH;
+        if (item < T1) {
+            slice = -1;
+            return item;
+        }
+        const int64_t j = item - T1, chunk = j / CH;
         slice = (int)(chunk % S);
-        return (chunk / S) * CH + item % CH;
+        return T1 + (chunk / S) * CH + j % CH;
     };
 
     // ---- loader ------------------------------------------------------------------------------------
@@ -141,6 +155,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     }
     uint32_t l_tail = 0;  // KTAIL: nonzero while the body being loaded is the one that holds the end of K
     if constexpr (KTAIL) asm volatile("s_mov_b32 %0, %1" : "=s"(l_tail) : "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kslice <= STREAM_K_MULTIPLE))));
+    uint32_t l_kbytes = kwhole_bytes;  // extent along K, in bytes, of the item being loaded
     const uint32_t dst_w = ring_base + (uint32_t)wave * 1024u;
     i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // empty descriptors: loads read zeros
     uint32_t l_koff = 0;  // byte offset along K of the body being loaded
@@ -152,24 +167,26 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
             const int row_a = __builtin_amdgcn_readfirstlane(rc.row * TILE), row_b = __builtin_amdgcn_readfirstlane(rc.col * TILE_N);
             const int ra = g.M - row_a < TILE ? g.M - row_a : TILE, rb = g.N - row_b < TILE_N ? g.N - row_b : TILE_N;
-            const int64_t k0 = (int64_t)slice * kslice_bytes;  // the slice starts k0 bytes into every row
+            const int64_t k0 = slice < 0 ? 0 : (int64_t)slice * kslice_bytes;  // the slice starts k0 bytes into every row
+            l_kbytes = slice < 0 ? kwhole_bytes : kslice_bytes;
             // (the descriptor's extent is counted from the shifted base: the last row ends k0 bytes early)
             rsrc_a = make_rsrc((const char*)g.A + (int64_t)row_a * pitch32 + k0, (uint32_t)ra * pitch32 - (uint32_t)k0);
             rsrc_b = make_rsrc((const char*)g.Bt + (int64_t)row_b * pitch32 + k0, (uint32_t)rb * pitch32 - (uint32_t)k0);
         } else {
             rsrc_a[2] = 0;  // past the last tile: nothing is fetched (the ring receives zeros nobody reads)
             rsrc_b[2] = 0;
+            l_kbytes = kwhole_bytes;
         }
     };
     auto loader_advance = [&]() __attribute__((always_inline)) {
         l_koff += STREAM_K_MULTIPLE * 2;
-        if (l_koff >= kslice_bytes) {
+        if (l_koff >= l_kbytes) {
             l_koff = 0;
             ++l_tile;
             loader_open_tile();
         }
         if constexpr (KTAIL)   // (kept in one opaque scalar register, like stores_in_flight below)
-            asm volatile("s_mov_b32 %0, %1" : "=s"(l_tail) : "s"(__builtin_amdgcn_readfirstlane((uint32_t)(l_koff + STREAM_K_MULTIPLE * 2 > kslice_bytes))));
+            asm volatile("s_mov_b32 %0, %1" : "=s"(l_tail) : "s"(__builtin_amdgcn_readfirstlane((uint32_t)(l_koff + STREAM_K_MULTIPLE * 2 > l_kbytes))));
     };
     // Load pair P (0, 1: A rows 16w.. / 16(w+8)..; 2, 3: Bt likewise; 256 x 128 tiles have no pair 3) of the body at l_koff: the two
     // halves of each row's line, back to back, into the quarters at byte offsets q_lo and q_hi.
@@ -314,26 +331,81 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < WTC; ++j) fb[0][j] = *(const CK_LDS u32x4*)(uintptr_t)(b_lane + (uint32_t)(j * 16 * RB));
 
-        for (int t = 0; t < my_tiles; ++t) {
-            for (int b = 0; b < nb; ++b) {
-                kstep(std::integral_constant<int, 0>{}, q1);
-                kstep(std::integral_constant<int, 1>{}, q2);
-                loader_advance();
-                asm volatile("s_mov_b32 %0, 0" : "=s"(stores_in_flight));
-                // two quarters on: q0 <- q2, q1 <- q3 = q4 - QB (mod ring), q2 <- q4, q4 <- q1
-                {
-                    const uint32_t n0 = q2, n2 = q4, n4 = q1;
-                    uint32_t n1 = q2 + QB;
-                    if (n1 == (uint32_t)(NQ * QB)) n1 = 0;
-                    q0 = n0; q1 = n1; q2 = n2; q4 = n4;
+        // K slices reduced in the kernel. Each wave handles its own wave tile of D, which S waves hold one slice of:
+        // the wave of slice s owns the accumulator block rows i with i % S == s. It stores its other rows to scratch
+        // memory in the accumulators' own layout (1 KiB per store), announces them, waits until all S waves have
+        // announced, adds what the others stored for its rows to its accumulators - its own slice first, then the
+        // others in slice order, a fixed order per element - and runs the ordinary epilogue on its rows only. The S
+        // waves wait for one another, so they must all be running: the host cuts tiles this way only when every
+        // workgroup gets at most one sliced item (its last) and there are no more workgroups than the device has CUs.
+        auto reduce_slices = [&](int64_t tc, int slice) __attribute__((always_inline)) {
+            unsigned own_rows = 0;
+            // The stored rows cross from one XCD's CU to another's, and the L2s of different XCDs do not see each
+            // other's lines. Fences would make that safe by writing back and invalidating whole L2s, once per
+            // wave (measured: 45 us per launch); instead the rows are stored and loaded with system-scope
+            // accesses (sc0 sc1: written through to memory, read past both caches), the announcement follows the
+            // completion of the stores, and no cache is touched as a whole.
+            constexpr int ROW_BYTES = WTC * 1024;          // one block row of a wave tile: 16 bytes per lane and block
+            constexpr int SYSTEM_SCOPE = 1 | 16;           // sc0 | sc1 of a buffer access
+            const int unit = __builtin_amdgcn_readfirstlane((int)(tc - T1) * 8 + wave);
+            // (one counter per 128-byte line: thousands of waves poll them, and counters that share a line share a memory channel)
+            unsigned int* announced = g.fix_state + (size_t)unit * (FIX_STATE_STRIDE_BYTES / 4);
+            // per (tile, wave): [block row][contributor: the S - 1 slices that do not own the row, in slice order]
+            const int unit_bytes = WTR * (S - 1) * ROW_BYTES;
+            const __amdgpu_buffer_rsrc_t rows = __builtin_amdgcn_make_buffer_rsrc((char*)g.fix_partials + (size_t)unit * (size_t)unit_bytes, 0,
+                                                                                  unit_bytes, 0x00020000);
+            const int ln16 = lane * 16;
+            own_rows = 0;
+#pragma unroll
+            for (int i = 0; i < WTR; ++i) {
+                const int owner = i % S;
+                if (owner == slice) {
+                    own_rows |= 1u << i;
+                } else {
+                    const int at = __builtin_amdgcn_readfirstlane((i * (S - 1) + (slice < owner ? slice : slice - 1)) * ROW_BYTES);
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j)
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rows, ln16, at + j * 1024, SYSTEM_SCOPE);
                 }
             }
-            // D = alpha * acc + beta * C straight from the accumulators
-            int slice = 0;
-            const int64_t tc = item_tile(slot + (int64_t)t * grid, slice);
+            own_rows = __builtin_amdgcn_readfirstlane(own_rows);
+            // the stores are complete (in memory) before the announcement
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (lane == 0) __hip_atomic_fetch_add(announced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (uint32_t n = 0;; ++n) {
+                const uint32_t seen = __builtin_amdgcn_readfirstlane(__hip_atomic_load(announced, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                if ((int)seen >= S) break;
+                if (n > g.spin_limit) {   // the grid drains whatever happens; the status word says D is invalid
+                    if (lane == 0) atomicOr(g.status, CK_STATUS_REDUCTION_TIMEOUT);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(8);
+            }
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int i = 0; i < WTR; ++i) {
+                if (own_rows & (1u << i)) {
+                    // one contributor after the other, in slice order (deeper queues - two or three contributors' loads in
+                    // flight - measured no faster: what this phase costs is the wait for the slowest slice, not the loads)
+                    for (int c = 0; c < S - 1; ++c) {
+                        const int at = __builtin_amdgcn_readfirstlane((i * (S - 1) + c) * ROW_BYTES);
+                        u32x4 x[WTC];
+#pragma unroll
+                        for (int j = 0; j < WTC; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b128(rows, ln16, at + j * 1024, SYSTEM_SCOPE);
+#pragma unroll
+                        for (int j = 0; j < WTC; ++j) acc[i][j] += __builtin_bit_cast(f32x4, x[j]);
+                    }
+                }
+            }
+            return own_rows;
+        };
+        // D = alpha * acc + beta * C for the block rows `own_rows` of this wave's wave tile, straight from the accumulators;
+        // returns whether the tile is an interior one (every wave then issues exactly the stores the next body's landing wait counts)
+        auto write_tile = [&](int64_t tc, int slice, unsigned own_rows) __attribute__((always_inline)) {
+            const bool sliced = slice >= 0;
             const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
-            GemmArgs go = g;  // a K slice writes its own plane of the workspace D points at
-            go.D = g.D + (size_t)slice * ((size_t)g.M * g.N);
+            GemmArgs go = g;  // without the reduction in the kernel a K slice writes its own plane of the workspace D points at
+            if (sliced && g.fix_partials == nullptr) go.D = g.D + (size_t)slice * ((size_t)g.M * g.N);
             const int m_base = rc.row * TILE + R * WTR * 16 + (int)(threadIdx.x & 15);
             const int n_base = rc.col * TILE_N + Cc * WTC * 16 + (int)((threadIdx.x >> 4) & 3) * 4;
             // vec_cols: every column of the tile is inside the matrix, one vector access per block (rows past M are
@@ -383,7 +455,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                             for (int tt = 0; tt < STORES_PER_GROUP; ++tt) {
                                 const f32x4 v = exchanged(i, j, tt);
                                 const int64_t row = row0 + i * 16 + tt * 8;
-                                if (row < g.M) put(row * g.N + (col0 + j * 16), v);
+                                if (row < g.M && (own_rows & (1u << i))) put(row * g.N + (col0 + j * 16), v);
                             }
                         }
                     }
@@ -392,7 +464,10 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                     // by one between the stores (a load may not pass the store in front of it)
                     constexpr int C_DEPTH = 4;
                     f32x4 cv[C_DEPTH];
-                    auto row_of = [&](int st) { return row0 + (st / (GROUPS * STORES_PER_GROUP)) * 16 + (st % STORES_PER_GROUP) * 8; };
+                    auto row_of = [&](int st) {   // (a block row another slice's wave writes counts as past the edge)
+                        return (own_rows & (1u << (st / (GROUPS * STORES_PER_GROUP)))) ? row0 + (st / (GROUPS * STORES_PER_GROUP)) * 16 + (st % STORES_PER_GROUP) * 8
+                                                                                     : (int64_t)g.M;
+                    };
                     auto off_of = [&](int st) { return row_of(st) * g.N + (col0 + ((st / STORES_PER_GROUP) % GROUPS) * F32_GROUP * 16); };
                     auto fetch = [&](int st) __attribute__((always_inline)) {
                         return row_of(st) < g.M ? (f32x4)*(const f32x4_u*)(go.C + off_of(st)) : f32x4{0.f, 0.f, 0.f, 0.f};
@@ -460,6 +535,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                     for (int j = 0; j < WTC; j += H16_GROUP) {
                         const int gi = i * GROUPS16 + j / H16_GROUP;   // this group; the next one's C goes into the other buffer
                         if (gi + 1 < WTR * GROUPS16) fetch_c((gi + 1) / GROUPS16, ((gi + 1) % GROUPS16) * H16_GROUP, cq[(gi + 1) % 2]);
+                        if (!(own_rows & (1u << i))) continue;   // a block row another slice's wave writes
                         const u32x4 first = packed_pair(scaled(acc[i][j], cq[gi % 2][0]), scaled(acc[i][j + 1], cq[gi % 2][1]));
                         const u32x4 second = packed_pair(scaled(acc[i][j + 2], cq[gi % 2][2]), scaled(acc[i][j + 3], cq[gi % 2][3]));
                         u32x4 other;  // the second pair's piece of the row 8 away
@@ -482,8 +558,35 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
                 for (int i = 0; i < WTR; ++i)
 #pragma unroll
-                    for (int j = 0; j < WTC; ++j) epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], vec_cols);
+                    for (int j = 0; j < WTC; ++j)
+                        if (own_rows & (1u << i)) epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], vec_cols);
             }
+            return interior;
+        };
+        for (int t = 0; t < my_tiles; ++t) {
+            int slice = 0;
+            const int64_t tc = item_tile(slot + (int64_t)t * grid, slice);
+            const bool sliced = slice >= 0;
+            const int nb = sliced ? nb_slice : nb_whole;
+            for (int b = 0; b < nb; ++b) {
+                kstep(std::integral_constant<int, 0>{}, q1);
+                kstep(std::integral_constant<int, 1>{}, q2);
+                loader_advance();
+                asm volatile("s_mov_b32 %0, 0" : "=s"(stores_in_flight));
+                // two quarters on: q0 <- q2, q1 <- q3 = q4 - QB (mod ring), q2 <- q4, q4 <- q1
+                {
+                    const uint32_t n0 = q2, n2 = q4, n4 = q1;
+                    uint32_t n1 = q2 + QB;
+                    if (n1 == (uint32_t)(NQ * QB)) n1 = 0;
+                    q0 = n0; q1 = n1; q2 = n2; q4 = n4;
+                }
+            }
+            unsigned own_rows = (1u << WTR) - 1;   // block rows of the wave tile this wave writes to D
+            const bool reduce_here = !KTAIL && sliced && g.fix_partials != nullptr;
+            if constexpr (!KTAIL) {
+                if (reduce_here) own_rows = reduce_slices(tc, slice);
+            }
+            const bool interior = write_tile(tc, slice, own_rows) && !reduce_here;
 #pragma unroll
             for (int i = 0; i < WTR; ++i)
 #pragma unroll

@@ -43,7 +43,9 @@ enum {
  * D = alpha * A * Bt^T + beta * C (textbook form; C is not read when beta == 0).
  * A: M x K row-major, Bt: N x K row-major (B transposed), dtype CKOPT_DT_F16 or CKOPT_DT_BF16;
  * C, D: M x N row-major fp32, distinct buffers (C may be NULL when beta == 0).
- * tile_dim in {64,128,256}; segment_dim_k in {32,64,128}; bar_step_rows_{a,b} select the
+ * tile_dim in {64,128,256}; segment_dim_k a multiple of 32 (the reference: of 64, port_2.cu:1113; port_0: of tile_dim / 2,
+ * port_0.cu:534), with kernel instances for 32, 64, 128 and - producer/consumer kernels on 64 and 128 tiles - 256; any other
+ * multiple is CKOPT_ERR_NO_INSTANCE (or CKOPT_ERR_LDS_BUDGET when one stage of it exceeds the LDS); bar_step_rows_{a,b} select the
  * synchronisation granularity exactly as in the reference: (tile_dim, tile_dim), or
  * (wave_tile_rows*16, wave_tile_cols*16) with bar_steps_a <= C/2 and bar_steps_b <= 2, or (16, 16)
  * with bar_steps_a < wave_tile_rows and bar_steps_b < wave_tile_cols; num_producer_waves in
@@ -88,7 +90,10 @@ int64_t ckopt_gemm_workspace_bytes(int M, int N, int K, int operands_aligned, in
 /* What a launch with these sizes and this tuning will run under the process's current options, without launching:
  * plan_out[0] = 1 if it takes the straight-line kernel (gemm_stream_kernel), 0 for the other designs;
  * plan_out[1] = width of its tiles in columns of D (256 or 128 for the straight-line kernel, else tile_dim);
- * plan_out[2] = number of K slices (1: no split-K); plan_out[3] = 1 if A and Bt are first copied into zero-padded rows.
+ * plan_out[2] = number of K slices (1: no split-K); plan_out[3] = 1 if A and Bt are first copied into zero-padded rows;
+ * plan_out[4] = number of tiles that are cut into those slices (all of them when there are fewer tiles than num_cus; the
+ * tiles of the partly filled last round otherwise; 0 without slices); plan_out[5] = 1 if the slices are added inside the
+ * kernel, 0 if by a second kernel; plan_out[6] = workgroups of the straight-line kernel's grid. plan_out points at 7 ints.
  * Returns CKOPT_OK or the error the launch would give. No reference counterpart (its launcher has one kernel form). */
 int ckopt_gemm_launch_plan(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b,
                            int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages, int num_producer_waves,
@@ -116,6 +121,52 @@ int ckopt_gemm_shmem_tc_async_opt_port_2_noalloc(int dtype, const void* A, const
                                                  int bar_step_rows_b, int tile_group_m, int num_stages,
                                                  int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
 
+/* Launch options as a per-call argument. In the reference every knob is a launcher parameter (port_2.cu:1088-1109);
+ * the knobs this implementation adds (kernel form, tile width, K slices, store policy, ...) are one struct here, so
+ * that a size query and the launch that follows it see the same values whatever other threads do, and two threads can
+ * launch with different settings at the same time. Each field has the meaning and range of the ckopt_set_option key
+ * named beside it; ckopt_launch_options_init fills the struct with the process-wide defaults (what ckopt_set_option
+ * last set), which are also what every entry point without an options argument uses - read once, at its start. */
+typedef struct ckopt_launch_options {
+    int struct_bytes;         /* sizeof(ckopt_launch_options): set by ckopt_launch_options_init, checked by the callee */
+    int lds_swizzle;          /* key 0 */
+    int spin_limit;           /* key 1 */
+    int num_xcd;              /* key 2 */
+    int prio_mode;            /* key 3 */
+    int producer_nap;         /* key 4 */
+    int tile_sync_barrier;    /* key 5 */
+    int straight_line;        /* key 6 */
+    int split_k;              /* key 7 */
+    int barrier_every_kstep;  /* key 8 */
+    int even_rounds;          /* key 9 */
+    int d_store_policy;       /* key 10 */
+    int half_width;           /* key 11 */
+    int tail_round;           /* key 12 */
+    int fused_reduction;      /* key 13 */
+} ckopt_launch_options;
+int ckopt_launch_options_init(ckopt_launch_options* options);
+
+/* The port_2 launcher (both C / D forms: cd_dtype CKOPT_DT_F32 or equal to dtype) with its options as an argument.
+ * options == NULL: the process-wide defaults. workspace == NULL: memory beyond the operands comes from stream-ordered
+ * allocations, as in ckopt_gemm_shmem_tc_async_opt_port_2; otherwise from [workspace, workspace + workspace_bytes), as
+ * in the _ws entry point, and nothing is allocated. ckopt_gemm_workspace_bytes_ex and ckopt_gemm_launch_plan_ex are
+ * the queries for the same arguments: query and launch are pure functions of what they are given (plus the device's
+ * compute-unit count, which the cost model reads once per device). No reference counterpart beyond port_2.cu:1088-1109. */
+int ckopt_gemm_shmem_tc_async_opt_port_2_ex(int dtype, int cd_dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim, int segment_dim_k,
+                                            int bar_steps_a, int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b,
+                                            int tile_group_m, int num_stages, int num_producer_waves, int num_consumer_waves,
+                                            int num_cus, const ckopt_launch_options* options, void* workspace,
+                                            size_t workspace_bytes, void* stream);
+int64_t ckopt_gemm_workspace_bytes_ex(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a,
+                                      int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
+                                      int num_producer_waves, int num_consumer_waves, int num_cus,
+                                      const ckopt_launch_options* options);
+int ckopt_gemm_launch_plan_ex(int M, int N, int K, int operands_aligned, int tile_dim, int segment_dim_k, int bar_steps_a,
+                              int bar_steps_b, int bar_step_rows_a, int bar_step_rows_b, int tile_group_m, int num_stages,
+                              int num_producer_waves, int num_consumer_waves, int num_cus, const ckopt_launch_options* options,
+                              int* plan_out);
+
 /* Replaces gemm_shmem_tc_async_opt_port<DT,DT_ACC>() of matmul_shmem_tc_async_opt_port_1.cu:889-965:
  * every wave tile (or every 16-row block) has its own signal, i.e. port_2 with maximal bar_steps. */
 int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* Bt, const float* C, float* D,
@@ -123,13 +174,25 @@ int ckopt_gemm_shmem_tc_async_opt_port_1(int dtype, const void* A, const void* B
                                          int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
                                          int tile_group_m, int num_stages, int num_producer_waves,
                                          int num_consumer_waves, int num_cus, void* stream);
+/* Its <half, half> instance (port_1.cu:1292, :1332): C and D in the operands' 16-bit type, as in the _2_lp entry point. */
+int ckopt_gemm_shmem_tc_async_opt_port_1_lp(int dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim,
+                                            int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
+                                            int tile_group_m, int num_stages, int num_producer_waves,
+                                            int num_consumer_waves, int num_cus, void* stream);
 
 /* Replaces gemm_shmem_tc_async_opt_port<DT,DT_ACC>() of matmul_shmem_tc_async_opt_port_0.cu:515-579:
- * one full/empty signal pair per operand and stage. */
+ * one full/empty signal pair per operand and stage. num_producer_waves may also be 1 (port_0.cu:538): the one wave
+ * streams the A rows and then the Bt rows of every segment (port_0.cu:106-147). */
 int ckopt_gemm_shmem_tc_async_opt_port_0(int dtype, const void* A, const void* Bt, const float* C, float* D,
                                          float alpha, float beta, int M, int N, int K, int tile_dim,
                                          int segment_dim_k, int tile_group_m, int num_stages,
                                          int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
+/* Its <half, half> instance (port_0.cu:866, :906). */
+int ckopt_gemm_shmem_tc_async_opt_port_0_lp(int dtype, const void* A, const void* Bt, const void* C, void* D,
+                                            float alpha, float beta, int M, int N, int K, int tile_dim,
+                                            int segment_dim_k, int tile_group_m, int num_stages,
+                                            int num_producer_waves, int num_consumer_waves, int num_cus, void* stream);
 
 /* Role of get_shmem_req<DT,DT_ACC>() (port_2.cu:1057-1086): dynamic LDS bytes of the launch, or a
  * negative error code. The caller may compare it with 160 KiB; the launcher does so itself. */
@@ -183,10 +246,10 @@ int ckopt_device_status(void* stream);
  * matrix-core utilisation. No reference counterpart. */
 int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* ref_ticks);
 
-/* Process-wide tuning switches that are not launcher parameters in the reference. Each is one atomic word that a
- * launch reads once; a switch changed by one thread while another launches takes effect for either all or none of
- * that launch, but two threads that need different settings at the same time must serialise their set / launch pairs
- * themselves (the reference's launchers have no such state: every knob there is a parameter).
+/* Process-wide defaults of the tuning switches that are not launcher parameters in the reference (ckopt_launch_options
+ * carries the same switches per call). An entry point without an options argument reads all of them once, when it
+ * starts: a switch changed by one thread while another launches takes effect for all or none of that launch. Two
+ * threads that need different settings at the same time use the _ex entry points.
  * key 0: LDS XOR swizzle on/off (default 1); key 1: spin limit of bounded waits (default 1<<22);
  * key 2: number of XCDs assumed by the workgroup->tile remap (default 8; 1 disables the remap);
  * key 3: wave priorities of the counter-synchronised kernel (0 producers raised (default), 1 also asymmetric
@@ -219,6 +282,18 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  *        0.86 of the rate on a full device) where the launcher's cost model gives them at least 5 % less time than
  *        256 x 256 tiles - tile counts that leave much of the device idle (2560^3: 100 tiles, 53 us -> 37 us);
  *        0: never; 2: always. tile_dim stays 256 in the launcher's parameters.
+ * key 12: the partly filled last round of the straight-line kernel (default 1). With more tiles than num_sms the last
+ *        round leaves CUs idle (6144^3: 576 tiles = 2 x 256 + 64); with 1 its tiles are cut into 2 to 4 K slices that
+ *        run as work items of the same launch behind the whole tiles, where the cost model gives that at least 3 % less
+ *        time than evenly filled rounds of whole tiles (key 9); needs keys 7 and 13 at 1. 0: never.
+ * key 13: where K slices are added. Inside the straight-line kernel: of every wave tile each slice's wave keeps some of
+ *        the accumulator block rows, stores the others to scratch memory ((slices - 1) x tile bytes and 1 KiB of counters
+ *        per cut tile), waits for the other slices' waves and adds what they stored for its rows, in a fixed order per
+ *        element (deterministic), and writes those rows of D; no second kernel. It needs every workgroup to hold at most
+ *        one sliced item (tiles x slices <= num_sms) and no more workgroups than the device has CUs. Or by a second
+ *        kernel over slices x M x N x 4 bytes of planes. 1 (default): inside the kernel where that is possible and the
+ *        cost model gives it less time (two slices of a large product: 18 us against 22; four slices of 2048 x 2048:
+ *        42 against 19, most of it the wait for the slowest slice); 2: wherever possible; 0: never.
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

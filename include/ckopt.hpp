@@ -5,6 +5,7 @@
 //                                             port_0:515-532 are the overloads with fewer parameters)
 //   matmul_shmem<DT,DT_ACC>                   matmul_shmem.cu:143-152
 //   get_shmem_req<DT,DT_ACC>                  port_2.cu:1057-1066        get_num_acc / get_warp_tile_rows  :158-169
+//   get_shmem_req<DT>(tile_dim)               matmul_shmem.cu:138-141
 //
 // DT is one of ckopt::half_t (IEEE fp16; layout-compatible with __half), ckopt::bfloat16_t, float, int;
 // DT_ACC is float (GEMM) or equals DT (matmul_shmem). Pointers are device memory owned by the caller.
@@ -100,21 +101,55 @@ void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B, const DT_ACC* C, DT_
                                   int K, int tile_dim, int segment_dim_k, int bar_step_rows_a, int bar_step_rows_b,
                                   int tile_group_m, int num_stages, int num_producer_warps, int num_consumer_warps, int num_sms,
                                   void* stream = nullptr) {
-    static_assert(std::is_same<DT_ACC, float>::value, "fp32 accumulate/output");
-    check(ckopt_gemm_shmem_tc_async_opt_port_1(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
-                                               bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
-                                               num_consumer_warps, num_sms, stream),
-          "gemm_shmem_tc_async_opt_port (port_1)");
+    static_assert(std::is_same<DT_ACC, float>::value || std::is_same<DT_ACC, DT>::value, "C / D are fp32 or the operand type");
+    if constexpr (std::is_same<DT_ACC, float>::value) {
+        check(ckopt_gemm_shmem_tc_async_opt_port_1(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
+                                                   bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages, num_producer_warps,
+                                                   num_consumer_warps, num_sms, stream),
+              "gemm_shmem_tc_async_opt_port (port_1)");
+    } else {  // the <half, half> instance (port_1.cu:1292, :1332)
+        check(ckopt_gemm_shmem_tc_async_opt_port_1_lp(dtype_of<DT>::value, A, B, C, D, to_float(alpha), to_float(beta), M, N, K, tile_dim,
+                                                      segment_dim_k, bar_step_rows_a, bar_step_rows_b, tile_group_m, num_stages,
+                                                      num_producer_warps, num_consumer_warps, num_sms, stream),
+              "gemm_shmem_tc_async_opt_port (port_1) <DT, DT>");
+    }
 }
 // port_0: one signal pair per stage
 template <typename DT, typename DT_ACC>
 void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B, const DT_ACC* C, DT_ACC* D, DT_ACC alpha, DT_ACC beta, int M, int N,
                                   int K, int tile_dim, int segment_dim_k, int tile_group_m, int num_stages,
                                   int num_producer_warps, int num_consumer_warps, int num_sms, void* stream = nullptr) {
-    static_assert(std::is_same<DT_ACC, float>::value, "fp32 accumulate/output");
-    check(ckopt_gemm_shmem_tc_async_opt_port_0(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
-                                               tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, stream),
-          "gemm_shmem_tc_async_opt_port (port_0)");
+    static_assert(std::is_same<DT_ACC, float>::value || std::is_same<DT_ACC, DT>::value, "C / D are fp32 or the operand type");
+    if constexpr (std::is_same<DT_ACC, float>::value) {
+        check(ckopt_gemm_shmem_tc_async_opt_port_0(dtype_of<DT>::value, A, B, C, D, alpha, beta, M, N, K, tile_dim, segment_dim_k,
+                                                   tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, stream),
+              "gemm_shmem_tc_async_opt_port (port_0)");
+    } else {  // the <half, half> instance (port_0.cu:866, :906)
+        check(ckopt_gemm_shmem_tc_async_opt_port_0_lp(dtype_of<DT>::value, A, B, C, D, to_float(alpha), to_float(beta), M, N, K, tile_dim,
+                                                      segment_dim_k, tile_group_m, num_stages, num_producer_warps, num_consumer_warps,
+                                                      num_sms, stream),
+              "gemm_shmem_tc_async_opt_port (port_0) <DT, DT>");
+    }
+}
+// port_2 with the launch options as an argument (ckopt_launch_options; nullptr: the process-wide defaults) and, optionally,
+// caller-owned scratch memory (nullptr: stream-ordered allocations)
+template <typename DT, typename DT_ACC>
+void gemm_shmem_tc_async_opt_port(const DT* A, const DT* B, const DT_ACC* C, DT_ACC* D, DT_ACC alpha, DT_ACC beta, int M, int N, int K,
+                                  int tile_dim, int segment_dim_k, int bar_steps_a, int bar_steps_b, int bar_step_rows_a,
+                                  int bar_step_rows_b, int tile_group_m, int num_stages, int num_producer_warps, int num_consumer_warps,
+                                  int num_sms, const ckopt_launch_options* options, void* workspace, std::size_t workspace_bytes,
+                                  void* stream) {
+    static_assert(std::is_same<DT_ACC, float>::value || std::is_same<DT_ACC, DT>::value, "C / D are fp32 or the operand type");
+    check(ckopt_gemm_shmem_tc_async_opt_port_2_ex(dtype_of<DT>::value, dtype_of<DT_ACC>::value, A, B, C, D, to_float(alpha), to_float(beta), M, N,
+                                                  K, tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b,
+                                                  tile_group_m, num_stages, num_producer_warps, num_consumer_warps, num_sms, options,
+                                                  workspace, workspace_bytes, stream),
+          "gemm_shmem_tc_async_opt_port (options)");
+}
+inline ckopt_launch_options default_launch_options() {
+    ckopt_launch_options o;
+    check(ckopt_launch_options_init(&o), "launch_options_init");
+    return o;
 }
 
 template <typename DT, typename DT_ACC>
@@ -128,6 +163,13 @@ int get_shmem_req(int tile_dim, int segment_dim_k, int bar_steps_a, int bar_step
                   int num_stages, int num_consumer_warps) {
     const int r = ckopt_get_lds_req(tile_dim, segment_dim_k, bar_steps_a, bar_steps_b, bar_step_rows_a, bar_step_rows_b, num_stages,
                                     num_consumer_warps);
+    if (r < 0) throw Error(r, "get_shmem_req");
+    return r;
+}
+// get_shmem_req<DT>(tile_dim) of matmul_shmem.cu:138-141: dynamic LDS bytes of a matmul_shmem launch
+template <typename DT>
+int get_shmem_req(int tile_dim) {
+    const int r = ckopt_matmul_shmem_lds_req(dtype_of<DT>::value, tile_dim);
     if (r < 0) throw Error(r, "get_shmem_req");
     return r;
 }
@@ -148,13 +190,18 @@ struct LaunchPlan {
     bool straight_line;
     int tile_cols, k_slices;
     bool operand_copies;
+    int sliced_tiles;          // tiles cut into k_slices (0: none)
+    bool reduced_in_kernel;    // the slices are added inside the kernel (no second kernel)
+    int grid;                  // workgroups of the straight-line kernel
 };
-inline LaunchPlan gemm_launch_plan(int M, int N, int K, bool operands_aligned, const Tuning& t, int num_sms) {
-    int v[4];
-    check(ckopt_gemm_launch_plan(M, N, K, operands_aligned ? 1 : 0, t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b, t.bar_step_rows_a,
-                                 t.bar_step_rows_b, t.tile_group_m, t.num_stages, t.num_producer_warps, t.num_consumer_warps, num_sms, v),
+inline LaunchPlan gemm_launch_plan(int M, int N, int K, bool operands_aligned, const Tuning& t, int num_sms,
+                                   const ckopt_launch_options* options = nullptr) {
+    int v[7];
+    check(ckopt_gemm_launch_plan_ex(M, N, K, operands_aligned ? 1 : 0, t.tile_dim, t.segment_dim_k, t.bar_steps_a, t.bar_steps_b,
+                                    t.bar_step_rows_a, t.bar_step_rows_b, t.tile_group_m, t.num_stages, t.num_producer_warps,
+                                    t.num_consumer_warps, num_sms, options, v),
           "gemm_launch_plan");
-    return LaunchPlan{v[0] != 0, v[1], v[2], v[3] != 0};
+    return LaunchPlan{v[0] != 0, v[1], v[2], v[3] != 0, v[4], v[5] != 0, v[6]};
 }
 
 inline int get_num_acc(int tile_dim, int num_consumer_warps) {

@@ -104,6 +104,62 @@ static int correctness(int cus) {
     return failed;
 }
 
+// The same closed form through the port_0 launcher over its own legal set (matmul_shmem_tc_async_opt_port_0.cu:515-540,
+// driver sweep :867): 1, 2, 4 and 8 producer warps, segment depths that are multiples of tile_dim / 2; and through the
+// <half, half> instances of the port_0 and port_1 launchers (port_0.cu:866, :906; port_1.cu:1292, :1332), whose results
+// 10 * dim + 1 are exact in fp16 up to dim 204.
+static int correctness_port_0(int cus) {
+    const int dim_max = 512;
+    const size_t n = (size_t)dim_max * dim_max;
+    std::vector<DT> a(n), b(n), c16(n), res16(n);
+    std::vector<DT_ACC> c(n), res(n);
+    ckopt::check(ckopt_fill_constant(CKOPT_DT_F16, a.data(), (int64_t)n, 1.f), "fill");
+    ckopt::check(ckopt_fill_constant(CKOPT_DT_F16, b.data(), (int64_t)n, 10.f), "fill");
+    ckopt::check(ckopt_fill_constant(CKOPT_DT_F32, c.data(), (int64_t)n, 1.f), "fill");
+    ckopt::check(ckopt_fill_constant(CKOPT_DT_F16, c16.data(), (int64_t)n, 1.f), "fill");
+    Device d(n);
+    DT *C16 = nullptr, *D16 = nullptr;
+    HIP_OK(hipMalloc((void**)&C16, n * sizeof(DT))); HIP_OK(hipMalloc((void**)&D16, n * sizeof(DT)));
+    HIP_OK(hipMemcpy(d.A, a.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.B, b.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.C, c.data(), n * sizeof(DT_ACC), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(C16, c16.data(), n * sizeof(DT), hipMemcpyHostToDevice));
+    int failed = 0, run = 0;
+    const int tiles[] = {64, 128}, cons[] = {4, 8}, prods[] = {1, 2, 4, 8};
+    for (int tile : tiles) for (int cw : cons) for (int p : prods) for (int sk = tile / 2; sk <= 128; sk *= 2) for (int stages = 1; stages <= 3; ++stages) {
+        // the caller's job, as in the reference's drivers (port_0.cu:642-645): only tuples whose ring fits the shared memory
+        if (sk < 32 || ckopt::get_shmem_req<DT, DT_ACC>(tile, sk, 0, 0, tile, tile, stages, cw) > 160 * 1024) continue;
+        const int dim = run % 3 == 0 ? dim_max : (1 + run % (dim_max / tile)) * tile;
+        HIP_OK(hipMemset(d.D, 0, n * sizeof(DT_ACC)));
+        ckopt::gemm_shmem_tc_async_opt_port<DT, DT_ACC>(d.A, d.B, d.C, d.D, 1.f, 1.f, dim, dim, dim, tile, sk, 1 + run % 4, stages, p, cw, cus);
+        HIP_OK(hipMemcpy(res.data(), d.D, n * sizeof(DT_ACC), hipMemcpyDeviceToHost));
+        const float want = 10.f * dim + 1.f;
+        bool ok = ckopt_device_status(nullptr) == 0;
+        for (size_t i = 0; ok && i < (size_t)dim * dim; ++i) ok = std::fabs(res[i] - want) <= 0.001f;
+        for (size_t i = (size_t)dim * dim; ok && i < n; ++i) ok = res[i] == 0.f;
+        ++run;
+        if (!ok) { ++failed; std::printf("FAILED port_0 dim %d (%d, %d, %d, %d, %d, %d)\n", dim, tile, sk, 1 + (run - 1) % 4, stages, p, cw); }
+    }
+    // <half, half>: alpha, beta, C and D in fp16
+    const int dim16 = 192;
+    for (int p : prods) for (int which = 0; which < 2; ++which) {
+        if (which == 1 && p == 1) continue;   // port_1 takes 2, 4 or 8 producer warps
+        HIP_OK(hipMemset(D16, 0, n * sizeof(DT)));
+        if (which == 0)
+            ckopt::gemm_shmem_tc_async_opt_port<DT, DT>(d.A, d.B, C16, D16, (DT)1.f, (DT)1.f, dim16, dim16, dim16, 64, 64, 2, 2, p, 4, cus);
+        else
+            ckopt::gemm_shmem_tc_async_opt_port<DT, DT>(d.A, d.B, C16, D16, (DT)1.f, (DT)1.f, dim16, dim16, dim16, 64, 64, 32, 32, 2, 2, p, 4, cus);
+        HIP_OK(hipMemcpy(res16.data(), D16, n * sizeof(DT), hipMemcpyDeviceToHost));
+        bool ok = ckopt_device_status(nullptr) == 0;
+        for (size_t i = 0; ok && i < (size_t)dim16 * dim16; ++i) ok = (float)res16[i] == 10.f * dim16 + 1.f;
+        ++run;
+        if (!ok) { ++failed; std::printf("FAILED <half, half> %s, %d producer warps\n", which ? "port_1" : "port_0", p); }
+    }
+    (void)hipFree(C16); (void)hipFree(D16);
+    std::printf("correctness, port_0 legal set and <half, half> of port_0 / port_1: %d launches, %d failed\n", run, failed);
+    return failed;
+}
+
 // uniform[-1,1) operands; number of elements with |cpu - gpu| > 0.1 (the reference's accuracy count) must be 0.
 // T is the element type (fp16 or bf16); M, N, K need not be multiples of anything.
 template <typename T>
@@ -227,7 +283,7 @@ int main(int argc, char** argv) {
     HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, 0));
     int failed = 0;
     try {
-        if (!std::strcmp(what, "correctness") || !std::strcmp(what, "all")) failed += correctness(cus);
+        if (!std::strcmp(what, "correctness") || !std::strcmp(what, "all")) failed += correctness(cus) + correctness_port_0(cus);
         if (!std::strcmp(what, "accuracy") || !std::strcmp(what, "all")) failed += accuracy(cus);
         if (!std::strcmp(what, "performance") || !std::strcmp(what, "all")) failed += performance(argc > 2 ? std::atoi(argv[2]) : 4096, cus);
     } catch (const ckopt::Error& e) {

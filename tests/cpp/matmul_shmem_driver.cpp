@@ -34,10 +34,12 @@ template <typename DT> static void fill(std::vector<DT>& v, uint64_t stream_id) 
 
 // (tile_dim, block_rows) pairs the launcher accepts: the reference's three conditions (threads per block, values per
 // thread, divisibility, matmul_shmem.cu:204-206) are ckopt_check_matmul_shmem_tuning here
-template <typename F> static void for_each_legal_pair(F f) {
+// and the tile's shared memory fits the device (get_shmem_req<DT>(tile_dim), matmul_shmem.cu:138-141, :198-200)
+template <typename DT, typename F> static void for_each_legal_pair(F f) {
     for (int tile_dim = 32; tile_dim <= 256; tile_dim *= 2)
         for (int block_rows = 1; block_rows <= tile_dim; block_rows *= 2)
-            if (ckopt_check_matmul_shmem_tuning(tile_dim, block_rows) == CKOPT_OK) f(tile_dim, block_rows);
+            if (ckopt_check_matmul_shmem_tuning(tile_dim, block_rows) == CKOPT_OK && ckopt::get_shmem_req<DT>(tile_dim) <= 160 * 1024)
+                f(tile_dim, block_rows);
 }
 
 template <typename DT> struct DeviceBuffers {
@@ -75,7 +77,7 @@ static int run_correctness(int dim_max, int num_reps, float atol) {
     int failed = 0;
     unsigned lcg = 2463534242u;
     for (int b_transposed = 0; b_transposed < 2; ++b_transposed) {   // 0: B is K x N as in the reference; 1: N x K
-        for_each_legal_pair([&](int tile_dim, int block_rows) {
+        for_each_legal_pair<DT>([&](int tile_dim, int block_rows) {
             bool ok = true;
             for (int rep = 0; rep < num_reps; ++rep) {
                 // the first repetition at the full size, the others at a random multiple of the tile (role of Rerand/GetMatDim)
@@ -110,7 +112,7 @@ static int run_performance(int dim, int num_reps) {
     HIP_OK(hipMemcpy(d.B, b.data(), n * sizeof(DT), hipMemcpyHostToDevice));
     hipEvent_t start, stop;
     HIP_OK(hipEventCreate(&start)); HIP_OK(hipEventCreate(&stop));
-    for_each_legal_pair([&](int tile_dim, int block_rows) {
+    for_each_legal_pair<DT>([&](int tile_dim, int block_rows) {
         if (dim % tile_dim) return;
         float ms = 0.f;
         ckopt::matmul_shmem<DT, DT>(d.A, d.B, d.C, dim, dim, dim, tile_dim, block_rows);

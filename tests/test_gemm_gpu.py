@@ -285,6 +285,56 @@ def test_port_0_and_port_1_entry_points(ck):
         assert ck.device_status() == 0 and bool(torch.equal(d, want))
 
 
+def _exact_case(ck, M, N, K, seed):
+    a = ck.fill_int(ck.DT_F16, (M, K), seed, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), seed, 1, -2, 2)
+    want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32)
+    return G.to_dev(a), G.to_dev(bt), want
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 384, 512), (700, 520, 1000), (1280, 1536, 256)])   # whole tiles; ragged in M, N and K; 120 tiles on 16 workgroups
+def test_port_0_legal_set_single_producer_and_low_precision(ck, M, N, K):
+    """port_0's own legal set: one producer warp (port_0.cu:538, one wave streams A then Bt of every segment), and the
+    <half, half> instance (port_0.cu:866, :906); also through the port_1 launcher (port_1.cu:1292). Exact on small integers."""
+    da, db, want = _exact_case(ck, M, N, K, 43)
+    cus = 16 if M * N > 1 << 20 else 256
+    for p, tile, sk, stages, c in ((1, 128, 64, 3, 4), (1, 64, 32, 4, 8), (1, 128, 128, 1, 8), (1, 256, 64, 2, 8), (8, 128, 64, 2, 8)):
+        d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        ck.gemm_shmem_tc_async_opt_port_0(ck.DT_F16, da, db, None, d, 1.0, 0.0, M, N, K, tile, sk, 3, stages, p, c, cus)
+        assert ck.device_status() == 0 and np.array_equal(d.cpu().numpy(), want), (p, tile, sk, stages, c)
+    h = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    for p in (1, 2):
+        h.zero_()
+        ck.gemm_shmem_tc_async_opt_port_0_lp(ck.DT_F16, da, db, None, h, 1.0, 0.0, M, N, K, 128, 64, 3, 2, p, 4, cus)
+        assert ck.device_status() == 0 and np.array_equal(h.cpu().numpy(), want.astype(np.float16))
+    for rows in (128, 64, 16):
+        h.zero_()
+        ck.gemm_shmem_tc_async_opt_port_1_lp(ck.DT_F16, da, db, None, h, 1.0, 0.0, M, N, K, 128, 64, rows, rows, 3, 2, 4, 4, cus)
+        assert ck.device_status() == 0 and np.array_equal(h.cpu().numpy(), want.astype(np.float16))
+        d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        ck.gemm_shmem_tc_async_opt_port_1(ck.DT_F16, da, db, None, d, 1.0, 0.0, M, N, K, 128, 64, rows, rows, 3, 2, 4, 4, cus)
+        assert ck.device_status() == 0 and np.array_equal(d.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 384, 1024), (200, 136, 1000)])
+def test_segments_256_deep(ck, M, N, K):
+    """segment_dim_k 256, the upper end of the reference drivers' sweep (port_2.cu:1520-1564): producer/consumer kernels
+    on 64 and 128 tiles, every synchronisation granularity; exact on small integers."""
+    da, db, want = _exact_case(ck, M, N, K, 47)
+    for tile, c, stages in ((128, 4, 1), (128, 8, 1), (64, 4, 2), (64, 8, 2)):
+        for mode, sa, sb in all_modes(ck, tile, c):
+            t = make_tuning(ck, tile, 256, stages, 2, c, mode, sa, sb)
+            if not legal(ck, t):
+                continue
+            d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, da, db, None, d, 1.0, 0.0, M, N, K, tile, 256, sa, sb, t["bar_step_rows_a"],
+                                            t["bar_step_rows_b"], 4, stages, 2, c, 256)
+            assert ck.device_status() == 0 and np.array_equal(d.cpu().numpy(), want), (tile, c, stages, mode, sa, sb)
+    with pytest.raises(ck.CkoptError) as e:   # a legal depth without an instance
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, da, db, None, d, 1.0, 0.0, M, N, K, 128, 192, 0, 0, 128, 128, 4, 1, 2, 4, 256)
+    assert e.value.code == ck.ERR_NO_INSTANCE
+
+
 def test_errors_with_device_pointers(ck):
     a = torch.zeros(1 << 16, dtype=torch.float16, device="cuda")
     d = torch.zeros(1 << 16, dtype=torch.float32, device="cuda")
@@ -773,6 +823,129 @@ def test_split_k_bit_exact(ck, M, N, K, slices, cus, dt_name):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("M,N,K,cus,opts", [
+    (2048, 4096, 4096, 256, dict(split_k=2)),            # 128 tiles, two slices: every workgroup one item
+    (512, 512, 8192, 256, dict(split_k=4)),              # 4 tiles x 4 slices: a wave owns one block row
+    (700, 520, 6144, 256, dict(split_k=3)),              # ragged tiles, three slices: slice 0 owns two block rows
+    (512, 768, 16384, 256, dict(split_k=16)),            # 6 tiles x 16 slices: slices 4 .. 15 own nothing
+    (1024, 1280, 8192, 16, dict()),                      # the partly filled last round: 16 whole tiles + 4 sliced, one launch
+    (2048, 1280, 4096, 16, dict()),                      # two full rounds + 8 sliced tiles
+    (1000, 640, 8192, 8, dict(half_width=2)),            # 256 x 128 tiles: 4 x 5 on 8 workgroups, ragged in M
+    (1400, 1200, 4096, 8, dict(tail_round=0)),
+])
+def test_slices_reduced_in_the_kernel_exact(ck, M, N, K, cus, opts):
+    """K slices added inside the straight-line kernel (no second kernel): fp32 and 16-bit output, with and without C, exact
+    on small integers; the same bits as the two-kernel form on random data (both add the slices of an element in a fixed
+    order, but not the same one, so the comparison there is within rounding of the sums)."""
+    t = _straight_line_tuning(ck, cus)
+    tup = tuple(t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
+                               "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms"))
+    a = ck.fill_int(ck.DT_F16, (M, K), 97, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 97, 1, -2, 2)
+    c = ck.fill_int(ck.DT_F32, (M, N), 97, 2, -3, 3)
+    prod = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float64)
+    da, db, dc = G.to_dev(a), G.to_dev(bt), G.to_dev(c)
+    dc16 = G.to_dev(c.astype(np.float16))
+    o = ck.launch_options(fused_reduction=2, **opts)   # 2: in the kernel wherever that is possible, whatever the cost model says
+    plan = ck.gemm_launch_plan(M, N, K, True, *tup, options=o)
+    if opts.get("tail_round", 1):
+        assert plan["sliced_tiles"] > 0 and plan["reduced_in_kernel"], plan
+    for rep_ in range(2):   # twice: the counters are cleared by every launch
+        d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, da, db, dc, d, 2.0, -1.0, M, N, K, *tup, options=o)
+        assert ck.device_status() == 0
+        assert np.array_equal(d.cpu().numpy(), (2.0 * prod - c).astype(np.float32)), plan
+    h = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F16, da, db, dc16, h, 1.0, 1.0, M, N, K, *tup, options=o)
+    assert ck.device_status() == 0
+    assert np.array_equal(h.cpu().numpy(), (prod + c).astype(np.float16)), plan
+    # on a caller-owned workspace of exactly the size the query gives, poisoned
+    need = ck.gemm_workspace_bytes(M, N, K, True, *tup, options=o)
+    ws = torch.full((max(need, 1),), 0xA5, dtype=torch.uint8, device="cuda")
+    d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, da, db, None, d, 1.0, 0.0, M, N, K, *tup, options=o, workspace=ws if need else None,
+                                       workspace_bytes=need)
+    assert ck.device_status() == 0 and np.array_equal(d.cpu().numpy(), prod.astype(np.float32))
+    if need > 256:
+        with pytest.raises(ck.CkoptError) as e:
+            ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, da, db, None, d, 1.0, 0.0, M, N, K, *tup, options=o, workspace=ws,
+                                               workspace_bytes=need - 257)
+        assert e.value.code == ck.ERR_TOO_LARGE
+
+
+def test_slices_reduced_in_the_kernel_against_the_second_pass(ck, oracle):
+    """Random fp16 data, 128 tiles in two slices: the two forms of the reduction agree to the last bits of an fp32 sum of two
+    terms in different order (they are equal: two terms have one order), and both are within tolerance of the oracle."""
+    M, N, K = 2048, 4096, 4096
+    t = _straight_line_tuning(ck, 256)
+    tup = tuple(t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
+                               "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms"))
+    a = ck.fill_uniform(ck.DT_F16, (M, K), 99, 0, -1.0, 1.0)
+    bt = ck.fill_uniform(ck.DT_F16, (N, K), 99, 1, -1.0, 1.0)
+    da, db = G.to_dev(a), G.to_dev(bt)
+    out = []
+    for fused in (2, 0):
+        o = ck.launch_options(split_k=2, fused_reduction=fused)
+        assert ck.gemm_launch_plan(M, N, K, True, *tup, options=o)["reduced_in_kernel"] == bool(fused)
+        d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, da, db, None, d, 1.0, 0.0, M, N, K, *tup, options=o)
+        assert ck.device_status() == 0
+        out.append(d.cpu().numpy())
+    assert np.array_equal(out[0], out[1])
+    ref = oracle.gemm(oracle.DT_F16, a, bt, rows=(0, 256))
+    assert_close(oracle, ref, out[0][:256])
+
+
+def test_two_host_threads_with_different_options(ck):
+    """Launch options are an argument of the _ex entry points (in the reference every knob is a launcher parameter,
+    port_2.cu:1088-1109): two host threads launch at the same time on their own streams with different options - one cuts
+    K and reduces in the kernel on 256 x 128 tiles, the other runs whole 256 x 256 tiles - and both get exact results,
+    whatever the process-wide switches are set to meanwhile."""
+    import threading
+    M, N, K = 1024, 1024, 4096
+    t = _straight_line_tuning(ck, 256)
+    tup = tuple(t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
+                               "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms"))
+    da, db, want = _exact_case(ck, M, N, K, 101)
+    variants = [ck.launch_options(split_k=4, half_width=2, fused_reduction=2), ck.launch_options(split_k=0, half_width=0)]
+    plans = [ck.gemm_launch_plan(M, N, K, True, *tup, options=o) for o in variants]
+    assert plans[0]["k_slices"] == 4 and plans[0]["tile_cols"] == 128 and plans[1]["k_slices"] == 1 and plans[1]["tile_cols"] == 256
+    errors = []
+
+    def worker(i):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+            for _ in range(40):
+                with torch.cuda.stream(stream):
+                    d.fill_(float("nan"))
+                ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, da, db, None, d, 1.0, 0.0, M, N, K, *tup, options=variants[i], stream=stream)
+                stream.synchronize()
+                if not np.array_equal(d.cpu().numpy(), want):
+                    errors.append("thread %d: wrong result" % i)
+                    return
+        except Exception as e:   # noqa: BLE001 - reported to the main thread
+            errors.append("thread %d: %r" % (i, e))
+
+    def flipper(stop):
+        while not stop.is_set():
+            for key in (ck.OPT_SPLIT_K, ck.OPT_HALF_WIDTH):
+                prev = ck.set_option(key, 0)
+                ck.set_option(key, prev)
+
+    stop = threading.Event()
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)] + [threading.Thread(target=flipper, args=(stop,))]
+    for th in threads:
+        th.start()
+    for th in threads[:2]:
+        th.join()
+    stop.set()
+    threads[2].join()
+    assert not errors, errors
+    assert ck.device_status() == 0
+
+
 @pytest.mark.parametrize("M,N,K", [(512, 512, 256), (700, 390, 1024), (1024, 768, 4096), (260, 1000, 200)])
 def test_half_width_tiles_exact(ck, M, N, K):
     """256 x 128 tiles of the straight-line kernel, forced: fp32 and 16-bit C / D (whole-line and element-wise epilogues),
@@ -856,7 +1029,9 @@ def test_automatic_split_k_of_128_tiles_exact(ck):
     for width, planes in ((0, 2), (1, 0)):
         prev = ck.set_option(ck.OPT_HALF_WIDTH, width)
         try:
-            assert ck.gemm_workspace_bytes(M, N, K, True, *order) == (planes * M * N * 4 + 256 if planes else 0)
+            # (two slices of this size are added inside the kernel: one tile of fp32 and eight counter lines per tile)
+            assert ck.gemm_workspace_bytes(M, N, K, True, *order) == (128 * (256 * 256 * 4 + 8 * 128) + 256 if planes else 0)
+            assert ck.gemm_launch_plan(M, N, K, True, *order)["k_slices"] == (planes if planes else 1)
             assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want), width
         finally:
             ck.set_option(ck.OPT_HALF_WIDTH, prev)
@@ -1017,6 +1192,23 @@ def test_16384_cubed_exact(ck):
     assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
     assert np.array_equal(d.astype(np.int64).sum(axis=0), bi @ ai.sum(axis=0))
     for r in (0, 8191, 16383):
+        assert np.array_equal(d[r], (ai[r] @ bi.T).astype(np.float32))
+
+
+def test_16384_cubed_alpha_beta_one_exact(ck):
+    """The reference driver's own performance case: 16384^3 with alpha = beta = 1 and a C tile read in the epilogue
+    (port_2.cu:1559-1564), on small integers: every element exact."""
+    M = N = K = 16384
+    t = suggested_tuning(ck, M, N, K)
+    a = ck.fill_int(ck.DT_F16, (M, K), 193, 0, -2, 2)
+    bt = ck.fill_int(ck.DT_F16, (N, K), 193, 1, -1, 1)
+    c = ck.fill_int(ck.DT_F32, (M, N), 193, 2, -100, 100)
+    d = G.run_gemm(ck, ck.DT_F16, a, bt, c, 1.0, 1.0, t=t)
+    d -= c                                                  # exact: all values are small integers
+    ai, bi = a.astype(np.int64), bt.astype(np.int64)
+    assert np.array_equal(d.astype(np.int64).sum(axis=1), ai @ bi.sum(axis=0))
+    assert np.array_equal(d.astype(np.int64).sum(axis=0), bi @ ai.sum(axis=0))
+    for r in (0, 255, 256, 8191, 16383):
         assert np.array_equal(d[r], (ai[r] @ bi.T).astype(np.float32))
 
 

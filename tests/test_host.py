@@ -82,6 +82,17 @@ def test_tuning_legality_mirrors_reference_asserts(ck):
     assert ok() == ck.OK
     assert ok(tile_dim=96, bar_step_rows_a=96, bar_step_rows_b=96) == ck.ERR_BAD_PARAM     # port_2.cu:1112
     assert ok(segment_dim_k=48) == ck.ERR_BAD_PARAM                                          # :1113
+    # every multiple of 64 is legal in the reference (port_2.cu:1113; its drivers sweep 64 -> 256, :1520-1564): depths
+    # without a kernel instance are "no instance", not "bad parameter"; 256 has instances on 64 and 128 tiles
+    assert ok(segment_dim_k=192, num_stages=1) == ck.ERR_NO_INSTANCE
+    assert ok(segment_dim_k=256, num_stages=1) == ck.OK                       # 128 tile, one stage: 1 KiB + 128 KiB
+    assert ok(segment_dim_k=256, num_stages=2) == ck.ERR_LDS_BUDGET
+    assert ok(tile_dim=64, bar_step_rows_a=64, bar_step_rows_b=64, segment_dim_k=256, num_stages=2) == ck.OK
+    assert ok(segment_dim_k=256, num_stages=1, num_producer_waves=0) == ck.ERR_NO_INSTANCE   # producer/consumer kernels only
+    assert ok(segment_dim_k=320, num_stages=1) == ck.ERR_LDS_BUDGET
+    assert ok(segment_dim_k=96, num_stages=1) == ck.ERR_NO_INSTANCE
+    assert ok(segment_dim_k=0) == ck.ERR_BAD_PARAM and ok(segment_dim_k=-64) == ck.ERR_BAD_PARAM
+    assert ok(num_producer_waves=1) == ck.ERR_BAD_PARAM      # one producer warp is legal in port_0 only (port_0.cu:538)
     assert ok(num_producer_waves=3) == ck.ERR_BAD_PARAM                                      # :1122
     assert ok(num_producer_waves=0) == ck.OK                 # fused variant (extension), tile granularity only
     assert ok(num_producer_waves=0, bar_step_rows_a=64, bar_step_rows_b=64) == ck.ERR_NO_INSTANCE
@@ -129,6 +140,28 @@ def test_launch_rejects_bad_arguments_before_touching_the_gpu(ck):
     with pytest.raises(ck.CkoptError) as e:  # A not even 2-byte aligned
         ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, 17, 16, None, 16, 1.0, 0.0, 256, 256, 256, **args)
     assert e.value.code == ck.ERR_ALIGNMENT
+    # port_0 takes one producer warp (port_0.cu:538): the tuple passes validation and the call stops at the null pointers;
+    # the port_1 / port_2 launchers do not (port_2.cu:1122)
+    p0 = dict(tile_dim=128, segment_dim_k=64, tile_group_m=4, num_stages=2, num_producer_warps=1, num_consumer_warps=4, num_sms=256)
+    for fn in (ck.gemm_shmem_tc_async_opt_port_0, ck.gemm_shmem_tc_async_opt_port_0_lp):
+        with pytest.raises(ck.CkoptError) as e:
+            fn(ck.DT_F16, None, None, None, None, 1.0, 0.0, 256, 256, 256, **p0)
+        assert e.value.code == ck.ERR_NULL
+        with pytest.raises(ck.CkoptError) as e:
+            fn(ck.DT_F16, None, None, None, None, 1.0, 0.0, 256, 256, 256, **dict(p0, num_producer_warps=3))
+        assert e.value.code == ck.ERR_BAD_PARAM
+    with pytest.raises(ck.CkoptError) as e:
+        ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, None, None, None, None, 1.0, 0.0, 256, 256, 256, **dict(args, num_producer_warps=1))
+    assert e.value.code == ck.ERR_BAD_PARAM
+    p1 = dict(tile_dim=128, segment_dim_k=64, bar_step_rows_a=64, bar_step_rows_b=64, tile_group_m=4, num_stages=2, num_producer_warps=2,
+              num_consumer_warps=4, num_sms=256)
+    for fn in (ck.gemm_shmem_tc_async_opt_port_1, ck.gemm_shmem_tc_async_opt_port_1_lp):
+        with pytest.raises(ck.CkoptError) as e:
+            fn(ck.DT_F16, None, None, None, None, 1.0, 0.0, 256, 256, 256, **p1)
+        assert e.value.code == ck.ERR_NULL
+        with pytest.raises(ck.CkoptError) as e:
+            fn(ck.DT_F16, None, None, None, None, 1.0, 0.0, 256, 256, 256, **dict(p1, num_producer_warps=1))
+        assert e.value.code == ck.ERR_BAD_PARAM
 
 
 def test_matmul_shmem_tuning_legality(ck):
@@ -198,7 +231,8 @@ def test_normal_and_int_generators(ck):
 
 def test_option_keys_reject_values_outside_their_range(ck):
     # process-wide switches: a bad value changes nothing and reports the error
-    for key, bad in ((ck.OPT_NUM_XCD, 0), (ck.OPT_PRIO_MODE, 3), (ck.OPT_PRODUCER_NAP, -1), (ck.OPT_SPLIT_K, 17), (ck.OPT_D_STORE_POLICY, 3), (ck.OPT_HALF_WIDTH, 3), (99, 1)):
+    for key, bad in ((ck.OPT_NUM_XCD, 0), (ck.OPT_PRIO_MODE, 3), (ck.OPT_PRODUCER_NAP, -1), (ck.OPT_SPLIT_K, 17), (ck.OPT_D_STORE_POLICY, 3), (ck.OPT_HALF_WIDTH, 3), (99, 1),
+                     (14, 1), (-1, 0), (ck.OPT_SPIN_LIMIT, 0)):
         with pytest.raises(ck.CkoptError):
             ck.set_option(key, bad)
     prev = ck.set_option(ck.OPT_SPLIT_K, 0)
@@ -231,6 +265,11 @@ def test_suggested_tunings_are_legal_and_follow_the_measured_rules(ck):
     assert picks(2048, 2048, 2048)["tile_dim"] == 128   # 64 tiles of 256 and K too shallow to cut four times
     assert picks(512, 512, 512)["tile_dim"] == 64       # config 1
     assert picks(8192, 8192, 8200) == straight          # any K: its end is masked in the kernel (or in the operand copies)
+    # K a multiple of 8 but not of 64 runs on K itself (no copies), where no slice count is legal: few tiles with such a K
+    # must be judged as one pass over 16 tiles, not as the slices a K padded to 8256 would allow
+    assert ck.gemm_launch_plan(1024, 1024, 8200, True, *(straight[k] for k in ("tile_dim", "segment_dim_k")), 0, 0, 256, 256, 4, 5, 0, 8, 256)["k_slices"] == 1
+    assert picks(1024, 1024, 8200)["tile_dim"] in (64, 128)
+    assert picks(1024, 1024, 8192) == straight
     prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
     try:
         assert picks(8192, 8192, 8192)["num_producer_warps"] == 2 and picks(8192, 8192, 8192)["tile_dim"] == 256
@@ -298,8 +337,11 @@ def test_workspace_query_follows_the_launcher_rules(ck):
     assert ck.gemm_workspace_bytes(1536, 1536, 8192, True, *straight) == 4 * 1536 * 1536 * 4 + 256
     # the automatic slice count follows the launcher's cost model: 128 tiles with a deep K are cut in two (256 items),
     # with K 4096 not at all (the reduction pass would cost more than the idle half of the CUs); 81 tiles in three;
-    # 144 tiles never (two slices would be 288 items: two rounds)
-    assert ck.gemm_workspace_bytes(2048, 4096, 16384, True, *straight) == 2 * 2048 * 4096 * 4 + 256
+    # 144 tiles never (two slices would be 288 items: two rounds). Two slices of a large product are added inside the
+    # kernel: per tile one tile of fp32 (what each slice's waves store of the rows they do not own) and eight 128-byte
+    # counter lines, instead of two M x N planes
+    assert ck.gemm_workspace_bytes(2048, 4096, 16384, True, *straight) == 128 * 8 * 128 + 128 * 256 * 256 * 4 + 256
+    assert ck.gemm_workspace_bytes(2048, 4096, 16384, True, *straight, options=ck.launch_options(fused_reduction=0)) == 2 * 2048 * 4096 * 4 + 256
     assert ck.gemm_workspace_bytes(2048, 4096, 4096, True, *straight) == 0
     assert ck.gemm_workspace_bytes(2304, 2304, 12288, True, *straight) == 3 * 2304 * 2304 * 4 + 256
     assert ck.gemm_workspace_bytes(3072, 3072, 8192, True, *straight) == 0
@@ -318,11 +360,27 @@ def test_launch_plan_reports_what_a_launch_will_run(ck):
     # pure host arithmetic: kernel form, tile width, K slices, operand copies - the launcher's own rules
     straight = (256, 32, 0, 0, 256, 256, 4, 5, 0, 8, 256)
     pc = (128, 64, 0, 0, 128, 128, 4, 2, 2, 4, 256)
-    assert ck.gemm_launch_plan(8192, 8192, 8192, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=1, operand_copies=False)
-    assert ck.gemm_launch_plan(2048, 2048, 32768, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=4, operand_copies=False)
-    assert ck.gemm_launch_plan(6143, 4097, 3071, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=1, operand_copies=True)
-    assert ck.gemm_launch_plan(2560, 2560, 2560, True, *straight) == dict(straight_line=True, tile_cols=128, k_slices=1, operand_copies=False)
-    assert ck.gemm_launch_plan(8192, 8192, 8192, False, *pc) == dict(straight_line=False, tile_cols=128, k_slices=1, operand_copies=True)
+    def plan(*a, **kw):
+        return ck.gemm_launch_plan(*a, **kw)
+    assert plan(8192, 8192, 8192, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=1, operand_copies=False, sliced_tiles=0,
+                                                           reduced_in_kernel=False, grid=256)
+    assert plan(2048, 2048, 32768, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=4, operand_copies=False, sliced_tiles=64,
+                                                            reduced_in_kernel=False, grid=256)
+    assert plan(2048, 4096, 16384, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=2, operand_copies=False, sliced_tiles=128,
+                                                            reduced_in_kernel=True, grid=256)
+    assert plan(6143, 4097, 3071, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=1, operand_copies=True, sliced_tiles=0,
+                                                           reduced_in_kernel=False, grid=208)
+    assert plan(2560, 2560, 2560, True, *straight) == dict(straight_line=True, tile_cols=128, k_slices=1, operand_copies=False, sliced_tiles=0,
+                                                           reduced_in_kernel=False, grid=200)
+    assert plan(8192, 8192, 8192, False, *pc) == dict(straight_line=False, tile_cols=128, k_slices=1, operand_copies=True, sliced_tiles=0,
+                                                      reduced_in_kernel=False, grid=0)
+    # the partly filled last round: 20 tiles on 16 workgroups with a deep K -> 16 whole tiles, then 4 tiles in K slices
+    # added inside the kernel, all in one launch of 16 workgroups; switched off: 2 rounds of 10
+    tail = (256, 32, 0, 0, 256, 256, 4, 5, 0, 8, 16)
+    p = plan(1024, 1280, 8192, True, *tail)
+    assert p["sliced_tiles"] == 4 and p["k_slices"] in (2, 3, 4) and p["reduced_in_kernel"] and p["grid"] == 16
+    p = plan(1024, 1280, 8192, True, *tail, options=ck.launch_options(tail_round=0))
+    assert p["sliced_tiles"] == 0 and p["k_slices"] == 1 and p["grid"] == 16 and p["tile_cols"] == 256
     prev = ck.set_option(ck.OPT_HALF_WIDTH, 0)
     try:
         assert ck.gemm_launch_plan(2560, 2560, 2560, True, *straight)["tile_cols"] == 256
@@ -344,3 +402,48 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 2
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_query_and_plan_are_pure_functions_of_their_arguments(ck):
+    """The _ex queries take the launch options as an argument (in the reference every knob is a launcher parameter,
+    port_2.cu:1088-1109): what they answer depends on that argument alone, whatever the process-wide switches say."""
+    straight = (256, 32, 0, 0, 256, 256, 4, 5, 0, 8, 256)
+    shapes = [(2048, 2048, 32768), (2048, 4096, 16384), (6143, 4097, 3071), (2560, 2560, 2560), (300, 520, 4090), (8192, 8192, 8192)]
+    variants = [dict(), dict(split_k=0), dict(split_k=2), dict(half_width=0), dict(half_width=2), dict(fused_reduction=0),
+                dict(straight_line=0), dict(even_rounds=0), dict(tail_round=0)]
+    frozen = [ck.launch_options(**v) for v in variants]       # taken while the process-wide switches have their defaults
+    want = [[(ck.gemm_workspace_bytes(*s, True, *straight, options=o), ck.gemm_launch_plan(*s, True, *straight, options=o)) for s in shapes]
+            for o in frozen]
+    assert len({repr(w) for w in want}) > 4                    # the options do matter
+    changed = [(ck.OPT_SPLIT_K, 0), (ck.OPT_HALF_WIDTH, 2), (ck.OPT_STRAIGHT_LINE, 0), (ck.OPT_FUSED_REDUCTION, 0), (ck.OPT_EVEN_ROUNDS, 0)]
+    prev = [ck.set_option(k, v) for k, v in changed]
+    try:
+        got = [[(ck.gemm_workspace_bytes(*s, True, *straight, options=o), ck.gemm_launch_plan(*s, True, *straight, options=o)) for s in shapes]
+               for o in frozen]
+        assert got == want
+        # no options argument: the process-wide switches
+        assert ck.gemm_launch_plan(8192, 8192, 8192, True, *straight)["straight_line"] is False
+        assert ck.gemm_workspace_bytes(2048, 2048, 32768, True, *straight) == 0
+        # ckopt_launch_options_init reads them
+        assert ck.launch_options().split_k == 0 and ck.launch_options().half_width == 2
+    finally:
+        for (k, _), v in zip(changed, prev):
+            ck.set_option(k, v)
+    assert ck.launch_options().split_k == 1 and ck.launch_options().straight_line == 1
+    # a struct of another size, or a field outside its key's range, is refused
+    bad = ck.launch_options()
+    bad.struct_bytes = 8
+    with pytest.raises(ck.CkoptError) as e:
+        ck.gemm_workspace_bytes(2048, 2048, 32768, True, *straight, options=bad)
+    assert e.value.code == ck.ERR_BAD_PARAM
+    bad = ck.launch_options()
+    bad.split_k = 17
+    with pytest.raises(ck.CkoptError) as e:
+        ck.gemm_launch_plan(2048, 2048, 32768, True, *straight, options=bad)
+    assert e.value.code == ck.ERR_BAD_PARAM
+    with pytest.raises(ck.CkoptError) as e:   # the launch refuses it too, before any pointer is looked at
+        ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, None, None, None, None, 1.0, 0.0, 256, 256, 256, *straight, options=bad)
+    assert e.value.code == ck.ERR_BAD_PARAM
+    with pytest.raises(ck.CkoptError) as e:
+        ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, None, None, None, None, 1.0, 0.0, 256, 256, 256, *straight, options=ck.launch_options())
+    assert e.value.code == ck.ERR_NULL
