@@ -86,6 +86,113 @@ def valu_ceiling(random_operands, iters=400000):
     return out.value
 
 
+HWMON_GLOB = "/sys/class/drm/card*/device/hwmon/hwmon*"
+
+
+class PowerSampler:
+    """Board power of the first GPU from the amdgpu hwmon files (power1_input, microwatts; power1_cap is the limit in
+    force), sampled by a thread every few milliseconds while `running` is set. Where the files cannot be read the
+    sampler reports that and nothing else."""
+
+    def __init__(self, period_s=0.005):
+        import glob
+        import threading
+        self.period_s = period_s
+        self.path = None
+        self.cap_w = None
+        for d in sorted(glob.glob(HWMON_GLOB)):
+            f = os.path.join(d, "power1_input")
+            if os.path.exists(f) and os.access(f, os.R_OK):
+                self.path = f
+                try:
+                    self.cap_w = int(open(os.path.join(d, "power1_cap")).read()) / 1e6
+                except (OSError, ValueError):
+                    self.cap_w = None
+                break
+        self.samples = []          # (label, watts)
+        self.label = None
+        self._stop = threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True) if self.path else None
+        if self._thread:
+            self._thread.start()
+
+    def read_w(self):
+        try:
+            return int(open(self.path).read()) / 1e6
+        except (OSError, ValueError, TypeError):
+            return None
+
+    def _run(self):
+        while not self._stop.is_set():
+            label = self.label
+            if label is not None:
+                w = self.read_w()
+                if w is not None:
+                    self.samples.append((label, w))
+            time.sleep(self.period_s)
+
+    def stop(self):
+        self._stop.set()
+        if self._thread:
+            self._thread.join()
+
+    def summary(self, label):
+        ws = sorted(w for l, w in self.samples if l == label)
+        if not ws:
+            return None
+        return {"samples": len(ws), "mean_w": round(sum(ws) / len(ws), 1), "median_w": round(ws[len(ws) // 2], 1), "max_w": round(ws[-1], 1)}
+
+
+def power_report(ck, torch, cus, stream):
+    """--power: board power, the power limit in force and the shader clock while the device runs (1) the headline GEMM on
+    its random operands, (2) the same launches on constant operands, (3) the bare inner loop of the same tile shape on
+    random operands - each for about two seconds, after half a second of the same load. One JSON line."""
+    M = N = K = 8192
+    tup = ck.suggest_gemm_tuning(M, N, K, cus)
+    order = [tup[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
+                              "num_stages", "num_producer_warps", "num_consumer_warps")] + [cus]
+    dd = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    sampler = PowerSampler()
+    out = {"power_report": "fp16 8192^3, tuple %s" % (order,), "hwmon": sampler.path, "power_cap_w": sampler.cap_w,
+           "idle_w": sampler.read_w() if sampler.path else None, "cases": {}}
+    if not sampler.path:
+        out["note"] = "no readable power1_input under %s: board power is not observable from this process" % HWMON_GLOB
+    flops = 2.0 * M * N * K
+
+    def gemm_case(name, a, b):
+        da, db = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+        step = lambda: ck.gemm_shmem_tc_async_opt_port(ck.DT_F16, da, db, None, dd, 1.0, 0.0, M, N, K, *order, stream)
+        for _ in range(600):      # about half a second of the same load first
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        sampler.label = name
+        e0.record(stream)
+        for _ in range(2500):
+            step()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        sampler.label = None
+        ms = e0.elapsed_time(e1) / 2500
+        cyc, ticks = ck.last_launch_clocks(stream)
+        out["cases"][name] = {"launches": 2500, "ms_per_launch": round(ms, 5), "tflops": round(flops / ms * 1e-9, 1),
+                              "shader_clock_mhz": round(cyc / ticks * 100.0, 1) if ticks else None, "board_power": sampler.summary(name)}
+
+    gemm_case("gemm_random_operands", ck.fill_uniform(ck.DT_F16, (M, K), 0xC0FFEE03, 0, -1.0, 1.0), ck.fill_uniform(ck.DT_F16, (N, K), 0xC0FFEE03, 1, -1.0, 1.0))
+    gemm_case("gemm_constant_operands", ck.fill_constant(ck.DT_F16, (M, K), 1.0), ck.fill_constant(ck.DT_F16, (N, K), 1.0))
+    mfma_ceiling(1, 1, 1000000)   # half a second of the bare loop first
+    sampler.label = "bare_inner_loop_random_operands"
+    tf = mfma_ceiling(1, 1, 4000000)
+    sampler.label = None
+    out["cases"]["bare_inner_loop_random_operands"] = {"tflops": round(tf, 1), "board_power": sampler.summary("bare_inner_loop_random_operands")}
+    sampler.stop()
+    if ck.device_status() != 0:
+        print("device status non-zero", file=sys.stderr)
+        return 4
+    print(json.dumps(out))
+    return 0
+
+
 def cpu_baseline(ck, kind, dtype, a, b, M, N, K, budget_s=12.0):
     """Times the CPU oracle on a bounded row sample of the same operands; returns the JSON object."""
     from oracle import oracle as o
@@ -272,6 +379,9 @@ def main():
                          "8=0: one barrier per loop body); repeatable")
     ap.add_argument("--no-vendor", action="store_true",
                     help="skip timing the vendor library's GEMM (hipBLASLt through torch.mm, fp32 output) on the same operands")
+    ap.add_argument("--power", action="store_true",
+                    help="board power (amdgpu hwmon), power limit and shader clock under the headline GEMM on random and on constant "
+                         "operands and under the bare inner loop; one JSON line")
     ap.add_argument("--no-settle", action="store_true",
                     help="skip the set-up launches that bring the device to its sustained clock before warm-up")
     ap.add_argument("--grid", action="store_true",
@@ -323,6 +433,8 @@ def main():
         options[int(k)] = int(v)
     if args.grid:
         return grid(ck, torch, cus, torch.cuda.current_stream())
+    if args.power:
+        return power_report(ck, torch, cus, torch.cuda.current_stream())
 
     if args.shape:
         sm, sn, sk = (int(v) for v in args.shape.split(","))
@@ -400,8 +512,24 @@ def main():
     # then holds (0.79 ms). Batches of about 25 ms of launches are repeated until two consecutive batches agree
     # within 1 % (at least 75 ms in all).
     settle = {"launches": 0, "first_batch_ms": None, "last_batch_ms": None}
+    # What a job of a few launches sees, before any of that: the first 21 launches of this process one by one. Launch 1
+    # carries the runtime's first-launch work; launches 2 to 21 run on a device that comes from idle (top clock, then the
+    # power controller's undershoot).
+    cold = {"first_launch_ms": None, "cold_first_20_ms": None}
+    sampler = PowerSampler()
+    if not args.no_settle:
+        cev = [torch.cuda.Event(enable_timing=True) for _ in range(22)]
+        cev[0].record(stream)
+        for i in range(21):
+            step()
+            cev[i + 1].record(stream)
+        torch.cuda.synchronize()
+        cold["first_launch_ms"] = round(cev[0].elapsed_time(cev[1]), 5)
+        cold["cold_first_20_ms"] = round(cev[1].elapsed_time(cev[21]) / 20.0, 5)
+        settle["launches"] += 21
     if not args.no_settle:
         sev0, sev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        sampler.label = "settle"
 
         def timed_batch(n):
             sev0.record(stream)
@@ -423,6 +551,7 @@ def main():
             if prev is not None and spent_ms >= 75.0 and abs(cur - prev) <= 0.01 * prev:
                 break
             prev = cur
+        sampler.label = None
 
     for _ in range(args.warmup):
         step()
@@ -449,11 +578,14 @@ def main():
     # (median, min, max of single launches), and the clock workgroup 0 of a launch actually ran at
     nper = max(5, min(args.steps, 50))
     pev = [torch.cuda.Event(enable_timing=True) for _ in range(nper + 1)]
+    sampler.label = "after"
     pev[0].record(stream)
     for i in range(nper):
         step()
         pev[i + 1].record(stream)
     torch.cuda.synchronize()
+    sampler.label = None
+    sampler.stop()
     per = sorted(pev[i].elapsed_time(pev[i + 1]) for i in range(nper))
     launch_ms = {"n": nper, "median": round(per[nper // 2], 5), "min": round(per[0], 5), "max": round(per[-1], 5)}
     shader_mhz = None
@@ -489,11 +621,13 @@ def main():
             print("parity check failed: %d elements outside tolerance" % nbad, file=sys.stderr)
             return 5
 
-    traffic = None
+    traffic, traffic_commit = None, None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         try:
-            traffic = json.load(open(tpath)).get(args.workload)
+            tj = json.load(open(tpath))
+            traffic = tj.get(args.workload)
+            traffic_commit = tj.get("_commit")
         except Exception:
             traffic = None
 
@@ -510,10 +644,20 @@ def main():
         "roofline": {"bound": "mfma" if bound_name == "mfma" else "valu", "achieved": round(achieved, 2), "peak": peak,
                      "unit": "TFLOP/s", "frac": round(achieved / peak, 4), "traffic": traffic,
                      "traffic_source": None if traffic is None else "recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
-                                       "command (profiles/hbm_traffic.json), not measured in this run",
+                                       "command (profiles/hbm_traffic.json, taken at commit %s), not measured in this run" % traffic_commit,
                      "kernel_ms": round(kern_ms, 5), "flops_per_launch": flops, "launch_ms": launch_ms,
-                     "shader_clock_mhz": shader_mhz},
-        "setup": {"settle": settle, "note": "set-up launches before warm-up, until the device holds its sustained clock"},
+                     "shader_clock_mhz": shader_mhz,
+                     # the same fraction against the peak at the clock the kernel actually ran at (nominal 2400 MHz): what the
+                     # schedule achieves; frac / frac_at_measured_clock is the clock's share of the gap
+                     "frac_at_measured_clock": None if not shader_mhz else round(achieved / (peak * shader_mhz / 2400.0), 4),
+                     "board_power": {"cap_w": sampler.cap_w, "set_up_launches": sampler.summary("settle"), "launches_after_timed_region": sampler.summary("after"),
+                                     "source": sampler.path or "no readable amdgpu hwmon power1_input",
+                                     "note": "the driver's reading follows the load over about a second: phases of tens of milliseconds read low; "
+                                             "`python bench.py --power` holds each load for seconds (profiles/power_config3.txt)"}},
+        "setup": {"settle": settle, "cold": cold, "effective_warmup_launches": settle["launches"] + args.warmup,
+                  "note": "set-up launches before warm-up, until the device holds its sustained clock; `cold` is what a fresh process sees: "
+                          "launch 1 alone, then the mean of launches 2 to 21 (value at that rate: %s TFLOP/s)"
+                          % (None if not cold["cold_first_20_ms"] else round(flops / cold["cold_first_20_ms"] * 1e-9, 1))},
     }
     if kind == "gemm" and args.workload == "config3_fp16_8192" and not args.no_ceiling:
         # what the bare inner loop of this tile shape sustains on this device with random operands and the
