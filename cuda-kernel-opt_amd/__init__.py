@@ -20,7 +20,8 @@ OK, ERR_BAD_PARAM, ERR_LDS_BUDGET, ERR_NO_INSTANCE, ERR_HIP, ERR_ALIGNMENT, ERR_
 OPT_SWIZZLE, OPT_SPIN_LIMIT, OPT_NUM_XCD, OPT_PRIO_MODE, OPT_PRODUCER_NAP, OPT_TILE_SYNC_BARRIER, OPT_STRAIGHT_LINE, OPT_SPLIT_K, OPT_BARRIER_EVERY_KSTEP = 0, 1, 2, 3, 4, 5, 6, 7, 8
 OPT_EVEN_ROUNDS = 9
 OPT_TAIL_ROUND = 12       # the partly filled last round of the straight-line kernel as K-sliced items of the same launch (default 1)
-OPT_FUSED_REDUCTION = 13  # 2 to 4 K slices are added inside the straight-line kernel (default 1); 0: by a second kernel
+OPT_FUSED_REDUCTION = 13  # K slices are added inside the straight-line kernel: 1 where possible and estimated cheaper (default), 2 wherever possible, 0 never
+OPT_BATCHED_EMPTY_READS = 14  # wave-tile granularity: producers read all "released" counters of a stage in one look (default 1)
 OPT_HALF_WIDTH = 11  # 256 x 128 tiles of the straight-line kernel: 0 never, 1 where the cost model prefers them (default), 2 always
 OPT_D_STORE_POLICY = 10  # 0: non-temporal stores of D where its rows lie on 128-byte lines (default), 1: always, 2: never
 
@@ -47,7 +48,7 @@ class LaunchOptions(ctypes.Structure):
     """ckopt_launch_options: the launch options as a per-call argument (fields = the ckopt_set_option keys in order)."""
     _fields_ = [(n, ctypes.c_int) for n in (
         "struct_bytes", "lds_swizzle", "spin_limit", "num_xcd", "prio_mode", "producer_nap", "tile_sync_barrier", "straight_line",
-        "split_k", "barrier_every_kstep", "even_rounds", "d_store_policy", "half_width", "tail_round", "fused_reduction")]
+        "split_k", "barrier_every_kstep", "even_rounds", "d_store_policy", "half_width", "tail_round", "fused_reduction", "batched_empty_reads")]
 
 
 _lib.ckopt_launch_options_init.restype = _i

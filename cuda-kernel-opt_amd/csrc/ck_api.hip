@@ -47,12 +47,13 @@ namespace {
 // The knobs that are not launcher parameters in the reference. A launch works on one Options value: the caller's
 // ckopt_launch_options, or a snapshot of the process-wide defaults taken once when the entry point starts.
 enum { OPT_SWIZZLE, OPT_SPIN_LIMIT, OPT_NUM_XCD, OPT_PRIO_MODE, OPT_PRODUCER_NAP, OPT_TILE_SYNC_BARRIER, OPT_STRAIGHT_LINE, OPT_SPLIT_K,
-       OPT_BARRIER_EVERY_KSTEP, OPT_EVEN_ROUNDS, OPT_D_STORE_POLICY, OPT_HALF_WIDTH, OPT_TAIL_ROUND, OPT_FUSED_REDUCTION, NUM_OPTIONS };
+       OPT_BARRIER_EVERY_KSTEP, OPT_EVEN_ROUNDS, OPT_D_STORE_POLICY, OPT_HALF_WIDTH, OPT_TAIL_ROUND, OPT_FUSED_REDUCTION, OPT_BATCHED_EMPTY_READS,
+       NUM_OPTIONS };
 struct OptionRule { int initial, lo, hi; };
 constexpr OptionRule OPTION_RULES[NUM_OPTIONS] = {
     {1, 0, 1}, {1 << 22, 1, 0x7fffffff}, {8, 1, 64}, {0, 0, 2}, {0, 0, 2}, {0, 0, 1}, {1, 0, 1}, {1, 0, 16},
-    {1, 0, 1}, {1, 0, 1}, {0, 0, 2}, {1, 0, 2}, {1, 0, 1}, {1, 0, 2}};
-std::atomic<int> g_option[NUM_OPTIONS] = {{1}, {1 << 22}, {8}, {0}, {0}, {0}, {1}, {1}, {1}, {1}, {0}, {1}, {1}, {1}};
+    {1, 0, 1}, {1, 0, 1}, {0, 0, 2}, {1, 0, 2}, {1, 0, 1}, {1, 0, 2}, {1, 0, 1}};
+std::atomic<int> g_option[NUM_OPTIONS] = {{1}, {1 << 22}, {8}, {0}, {0}, {0}, {1}, {1}, {1}, {1}, {0}, {1}, {1}, {1}, {1}};
 struct Options {
     int v[NUM_OPTIONS];
     int operator[](int key) const { return v[key]; }
@@ -517,6 +518,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
     a.spin_limit = (uint32_t)opt[OPT_SPIN_LIMIT];
     a.prio_mode = opt[OPT_PRIO_MODE];
     a.producer_nap = opt[OPT_PRODUCER_NAP];
+    a.batched_empty_reads = opt[OPT_BATCHED_EMPTY_READS];
     const int src = status_ptr_for_current_device(&a.status);
     if (src != CK_OK) return src;
 

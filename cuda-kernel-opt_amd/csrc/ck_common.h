@@ -225,10 +225,14 @@ CK_HD MicroTile simt_micro_tile(int accs) {
     }
     return m;
 }
+// Row pitch of the k-major LDS slices beyond tile_dim. (Pitches of tile_dim + 8, 12, 16, 20 and 36 measured the same as
+// this one on fp32 4096^3, 90 to 93 TFLOP/s: the two-dword LDS writes of a fetched chunk collide in half of the banks at
+// every one of them, and cost nothing that shows - the kernel is bound by the vector ALUs' clock under load.)
+constexpr int SIMT_PAD = 4;
 constexpr int SIMT_KT = 16;  // K depth of one LDS tile of the SIMT kernel
 CK_HD int simt_lds_req(int tile_dim, int elem_bytes) {
     // two operands x two buffers x KT x (tile_dim + pad) elements
-    return 2 * 2 * SIMT_KT * (tile_dim + 4) * elem_bytes;
+    return 2 * 2 * SIMT_KT * (tile_dim + SIMT_PAD) * elem_bytes;
 }
 CK_HD int check_simt_tuning(int tile_dim, int block_rows) {
     if (!(tile_dim == 32 || tile_dim == 64 || tile_dim == 128)) return CK_ERR_BAD_PARAM;

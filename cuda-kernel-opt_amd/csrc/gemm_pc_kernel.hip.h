@@ -82,6 +82,7 @@ struct GemmArgs {
     uint32_t spin_limit;
     int prio_mode;      // 0: producers at raised priority; 1: also asymmetric consumer burst priorities per SIMD pair; 2: none
     int producer_nap;   // s_sleep argument class of the producers' flag polling: 0 -> 1, 1 -> 4, 2 -> 16
+    int batched_empty_reads;  // wave-tile granularity: a producer wave reads all "empty" counters of its operand and stage once per segment
     unsigned int* status;  // device words: [0] OR of CK_STATUS_* bits, [2..3] shader cycles and [4..5] 100 MHz
                            // ticks workgroup 0 spent in the last launch (actual-clock evidence)
 };
@@ -200,6 +201,21 @@ __device__ __forceinline__ void flag_add_after_reads(uint32_t lds_addr) {
 __device__ __forceinline__ void flag_add(uint32_t lds_addr) {
     uint32_t one = 1;
     asm volatile("s_mov_b64 exec, 1\n\tds_add_u32 %0, %1\n\ts_mov_b64 exec, -1" ::"v"(lds_addr), "v"(one) : "memory");
+}
+
+// Up to five adjacent counters in one round trip to the LDS (the reads are issued back to back and waited for once):
+// what a producer wave of the wave-tile granularity looks at once per segment instead of polling every row block's
+// counter on its own.
+__device__ __forceinline__ void flag_load5(uint32_t lds_addr, int n, uint32_t (&out)[5]) {
+    uint32_t v0, v1, v2, v3, v4;
+    const uint32_t a1 = lds_addr + (n > 1 ? 4u : 0u), a2 = lds_addr + (n > 2 ? 8u : 0u), a3 = lds_addr + (n > 3 ? 12u : 0u),
+                   a4 = lds_addr + (n > 4 ? 16u : 0u);
+    asm volatile("ds_read_b32 %0, %5\n\tds_read_b32 %1, %6\n\tds_read_b32 %2, %7\n\tds_read_b32 %3, %8\n\tds_read_b32 %4, %9\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4)
+                 : "v"(lds_addr), "v"(a1), "v"(a2), "v"(a3), "v"(a4)
+                 : "memory");
+    out[0] = __builtin_amdgcn_readfirstlane(v0); out[1] = __builtin_amdgcn_readfirstlane(v1); out[2] = __builtin_amdgcn_readfirstlane(v2);
+    out[3] = __builtin_amdgcn_readfirstlane(v3); out[4] = __builtin_amdgcn_readfirstlane(v4);
 }
 
 // Counter read whose answer is needed later: a relaxed workgroup-scope atomic load compiles to a
@@ -395,6 +411,17 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
             const uint32_t st_base = ring_base + (uint32_t)stage * (2 * OPB) + (IS_A ? 0 : OPB);
             const int k0 = seg * SEGK;
             const bool fast = all_rows && k0 + SEGK <= g.K;
+            // wave-tile granularity: all "empty" counters of this operand and stage in one look (g.batched_empty_reads);
+            // a row block whose counter was already there is not polled again
+            uint32_t seen[5] = {0, 0, 0, 0, 0};
+            const bool batched = MODE == CK_SYNC_WAVE && g.batched_empty_reads && fill > 0;
+            if (MODE == CK_SYNC_WAVE) {
+                if (batched) flag_load5(fl + empty_off * 4, (IS_A ? sa : sb) + 1, seen);
+            }
+            auto wave_wait = [&](int idx, uint32_t target) __attribute__((always_inline)) {
+                if (batched && (int32_t)(seen[idx] - target) >= 0) return;
+                producer_wait(fl + (empty_off + idx) * 4, target, sq, sp, g.producer_nap);
+            };
 #pragma unroll
             for (int blk = 0; blk < NBLK; ++blk) {
                 // ---- wait until the consumers of the previous fill have released these rows
@@ -404,11 +431,11 @@ __device__ __forceinline__ void produce(const GemmArgs& g, uint32_t flags_base, 
                     const int s_own = IS_A ? sa : sb, s_oth = IS_A ? sb : sa;
                     const int oth_max = IS_A ? 2 : CW / 2;
                     const bool first_has_res = (s_own == 0 || s_oth < oth_max);
-                    if (blk == 0 && first_has_res && nres > 0) producer_wait(fl + (empty_off + s_own) * 4, nres * fill, sq, sp, g.producer_nap);
+                    if (blk == 0 && first_has_res && nres > 0) wave_wait(s_own, nres * fill);
                     if (blk < s_own && s_oth > 0) {
-                        producer_wait(fl + (empty_off + blk) * 4, s_oth * fill, sq, sp, g.producer_nap);
+                        wave_wait(blk, s_oth * fill);
                     } else if (blk == s_own && !first_has_res && nres > 0) {
-                        producer_wait(fl + (empty_off + s_own) * 4, nres * fill, sq, sp, g.producer_nap);
+                        wave_wait(s_own, nres * fill);
                     }
                 } else {
                     constexpr int WT = IS_A ? WTR : WTC;

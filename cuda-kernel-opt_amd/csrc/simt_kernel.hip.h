@@ -67,7 +67,7 @@ __global__ __launch_bounds__(TILE * TILE / (RM * RN)) void matmul_shmem_kernel(c
     constexpr int KT = SIMT_KT;
     constexpr int VEC = SimtIo<DT>::VEC;
     constexpr int NT = TILE * TILE / (RM * RN);   // threads
-    constexpr int LD = TILE + 4;                  // LDS row pitch (elements), k-major
+    constexpr int LD = TILE + SIMT_PAD;           // LDS row pitch (elements), k-major
     constexpr int TX = TILE / RN;                 // threads along N
     constexpr int CPRK = KT / VEC;                // 16-byte chunks per row of a row-major (rows x KT) slice
     constexpr int CH_RK = TILE * CPRK;            // chunks of such a slice

@@ -143,6 +143,7 @@ typedef struct ckopt_launch_options {
     int half_width;           /* key 11 */
     int tail_round;           /* key 12 */
     int fused_reduction;      /* key 13 */
+    int batched_empty_reads;  /* key 14 */
 } ckopt_launch_options;
 int ckopt_launch_options_init(ckopt_launch_options* options);
 
@@ -294,6 +295,10 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  *        kernel over slices x M x N x 4 bytes of planes. 1 (default): inside the kernel where that is possible and the
  *        cost model gives it less time (two slices of a large product: 18 us against 22; four slices of 2048 x 2048:
  *        42 against 19, most of it the wait for the slowest slice); 2: wherever possible; 0: never.
+ * key 14: wave-tile granularity of the counter-synchronised kernel (default 1). 1: a producer wave reads all "released"
+ *        counters of its operand and stage in one look per segment and polls a row block's counter only if that look
+ *        found it short; 0: it polls every row block's counter on its own, as the reference's producers wait on every
+ *        barrier in turn (port_2.cu:212-232).
  * Returns the previous value or CKOPT_ERR_BAD_PARAM. */
 int ckopt_set_option(int key, int value);
 

@@ -46,6 +46,15 @@ inline void synchronize_and_check(void* stream = nullptr) {
     if (st != 0) throw DeviceStatusError(st);
 }
 
+// A launcher call followed by that check, for callers that want the reference's blocking behaviour (its drivers
+// synchronise right behind every launch, port_2.cu:1241-1242) together with an error instead of a silently wrong D:
+//     ckopt::checked(stream, [&] { ckopt::gemm_shmem_tc_async_opt_port<DT, float>(A, B, C, D, ...); });
+template <typename Launch>
+inline void checked(void* stream, Launch&& launch) {
+    launch();
+    synchronize_and_check(stream);
+}
+
 inline float to_float(float x) { return x; }
 inline float to_float(half_t x) { return (float)x; }
 inline float to_float(bfloat16_t x) {

@@ -71,6 +71,10 @@ static void launch(const Device& d, float alpha, float beta, int dim, const Tupl
     ckopt::gemm_shmem_tc_async_opt_port<DT, DT_ACC>(d.A, d.B, d.C, d.D, alpha, beta, dim, dim, dim, t.tile_dim, t.segment_dim_k, t.bar_steps_a,
                                                      t.bar_steps_b, t.rows_a, t.rows_b, t.tile_group_m, t.num_stages, t.producers, t.consumers, cus);
 }
+// the same launch, waited for and checked: a bounded wait that was given up throws instead of leaving a wrong D behind
+static void launch_checked(const Device& d, float alpha, float beta, int dim, const Tuple& t, int cus) {
+    ckopt::checked(nullptr, [&] { launch(d, alpha, beta, dim, t, cus); });
+}
 
 // A = 1, B = 10, C = 1: every element of D is alpha * 10 * dim + beta (the reference's closed form)
 static int correctness(int cus) {
@@ -91,10 +95,14 @@ static int correctness(int cus) {
         lcg = lcg * 1664525u + 1013904223u;
         const int dim = (run % 4 == 0) ? dim_max : std::max(t.tile_dim, (int)((lcg >> 8) % (dim_max + 1)) / t.tile_dim * t.tile_dim);
         HIP_OK(hipMemset(d.D, 0, n * sizeof(DT_ACC)));
-        launch(d, 1.f, 1.f, dim, t, cus);
+        bool ok = true;
+        try {
+            launch_checked(d, 1.f, 1.f, dim, t, cus);
+        } catch (const ckopt::DeviceStatusError&) {
+            ok = false;
+        }
         HIP_OK(hipMemcpy(res.data(), d.D, n * sizeof(DT_ACC), hipMemcpyDeviceToHost));
         const float want = 10.f * dim + 1.f;
-        bool ok = ckopt_device_status(nullptr) == 0;
         for (size_t i = 0; ok && i < (size_t)dim * dim; ++i) ok = std::fabs(res[i] - want) <= 0.001f;
         for (size_t i = (size_t)dim * dim; ok && i < n; ++i) ok = res[i] == 0.f;
         ++run;

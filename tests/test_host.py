@@ -232,7 +232,7 @@ def test_normal_and_int_generators(ck):
 def test_option_keys_reject_values_outside_their_range(ck):
     # process-wide switches: a bad value changes nothing and reports the error
     for key, bad in ((ck.OPT_NUM_XCD, 0), (ck.OPT_PRIO_MODE, 3), (ck.OPT_PRODUCER_NAP, -1), (ck.OPT_SPLIT_K, 17), (ck.OPT_D_STORE_POLICY, 3), (ck.OPT_HALF_WIDTH, 3), (99, 1),
-                     (14, 1), (-1, 0), (ck.OPT_SPIN_LIMIT, 0)):
+                     (15, 1), (-1, 0), (ck.OPT_SPIN_LIMIT, 0)):
         with pytest.raises(ck.CkoptError):
             ck.set_option(key, bad)
     prev = ck.set_option(ck.OPT_SPLIT_K, 0)
