@@ -22,7 +22,7 @@ OPT_EVEN_ROUNDS = 9
 OPT_TAIL_ROUND = 12       # the partly filled last round of the straight-line kernel as K-sliced items of the same launch (default 1)
 OPT_FUSED_REDUCTION = 13  # K slices are added inside the straight-line kernel: 1 where possible and estimated cheaper (default), 2 wherever possible, 0 never
 OPT_BATCHED_EMPTY_READS = 14  # wave-tile granularity: producers read all "released" counters of a stage in one look (default 1)
-OPT_HALF_WIDTH = 11  # 256 x 128 tiles of the straight-line kernel: 0 never, 1 where the cost model prefers them (default), 2 always
+OPT_HALF_WIDTH = 11  # tile width of the straight-line kernel: 0 always 256 x 256, 1 what the cost model prefers (default), 2 always 256 x 128, 3 always 256 x 192
 OPT_D_STORE_POLICY = 10  # 0: non-temporal stores of D where its rows lie on 128-byte lines (default), 1: always, 2: never
 
 if not os.path.exists(LIB_PATH):

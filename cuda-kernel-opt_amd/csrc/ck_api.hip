@@ -20,8 +20,8 @@ CK_DECL_GEMM(launch_gemm_pc_bf16_m0) CK_DECL_GEMM(launch_gemm_pc_bf16_m1) CK_DEC
 #undef CK_DECL_GEMM
 hipError_t launch_gemm_pcb_f16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
 hipError_t launch_gemm_pcb_bf16(int tile, int segk, int cw, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const GemmArgs& a);
-hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, bool half_width);
-hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, bool half_width);
+hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, int tile_n);
+hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, int tile_n);
 bool gemm_stream_applies(const GemmArgs& a, int tile_dim, int segment_dim_k, int num_stages, int producer_waves, int consumer_waves);
 constexpr int STREAM_K_MULTIPLE_HOST = 64;  // K extent of one loop body of the straight-line kernel
 hipError_t launch_gemm_fused_f16(int tile, int segk, int cw, dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a);
@@ -52,7 +52,7 @@ enum { OPT_SWIZZLE, OPT_SPIN_LIMIT, OPT_NUM_XCD, OPT_PRIO_MODE, OPT_PRODUCER_NAP
 struct OptionRule { int initial, lo, hi; };
 constexpr OptionRule OPTION_RULES[NUM_OPTIONS] = {
     {1, 0, 1}, {1 << 22, 1, 0x7fffffff}, {8, 1, 64}, {0, 0, 2}, {0, 0, 2}, {0, 0, 1}, {1, 0, 1}, {1, 0, 16},
-    {1, 0, 1}, {1, 0, 1}, {0, 0, 2}, {1, 0, 2}, {1, 0, 1}, {1, 0, 2}, {1, 0, 1}};
+    {1, 0, 1}, {1, 0, 1}, {0, 0, 2}, {1, 0, 3}, {1, 0, 1}, {1, 0, 2}, {1, 0, 1}};
 std::atomic<int> g_option[NUM_OPTIONS] = {{1}, {1 << 22}, {8}, {0}, {0}, {0}, {1}, {1}, {1}, {1}, {0}, {1}, {1}, {1}, {1}};
 struct Options {
     int v[NUM_OPTIONS];
@@ -263,45 +263,48 @@ bool scratch_release(const Scratch& sc, void* piece, hipStream_t s) {
 int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D, float alpha, float beta, int M,
                 int N, int K, const ck::GemmTuning& t, const Options& opt, void* stream, int out16, Scratch sc);
 
-// Estimated duration (microseconds) of the straight-line kernel on `tiles` tiles (256 x 256, or 256 x 128 with
-// half_width) of an M x N product with K cut into S slices, plus what adding the slices costs when S > 1. The constants
+// Estimated duration (microseconds) of the straight-line kernel on `tiles` tiles of 256 x tile_n (256, 192 or 128) of an
+// M x N product with K cut into S slices, plus what adding the slices costs when S > 1. The constants
 // are measurements of one MI355X (256 CUs) on random operands: a loop body (64 of K) of a 256 x 256 tile takes 1.05 us
 // while at most half of the CUs multiply and the clock is free, and grows with the share of active CUs once the device is
 // power-limited (1.42 us with all of them); a 256 x 128 tile's body has half the MFMAs and takes 0.585 of that time
-// at the power-limited clock but no less than 0.69 us (one barrier per 16 MFMAs); a work item costs about 3 us of pipeline
+// at the power-limited clock but no less than 0.69 us (one barrier per 16 MFMAs), a 256 x 192 tile's three quarters of
+// the MFMAs and BODY_192 of the time, no less than BODY_192_MIN_US; a work item costs about 3 us of pipeline
 // fill and drain; the items of a round store their tile at the 4.6 TB/s the write path sustains. The slices are added
-// either by a reduction pass (reads S planes and writes D at 5.3 TB/s behind about 3 us of launch) or, `fused`, by the
-// last wave tile to arrive, which reads the S - 1 others at what one CU draws from memory (about 110 GB/s). device_cus is
-// the device's real CU count: the power-limit knee lies at half of it. The model is calibrated for a 256-CU gfx950.
-constexpr double HALF_WIDTH_BODY = 0.585, HALF_WIDTH_BODY_MIN_US = 0.69;
-double body_us_for(double active, bool half_width, int dev_cus) {
+// either by a reduction pass (reads S planes and writes D at 5.3 TB/s behind about 3 us of launch) or inside the kernel.
+// device_cus is the device's real CU count: the power-limit knee lies at half of it. The model is calibrated for a
+// 256-CU gfx950.
+constexpr double HALF_WIDTH_BODY = 0.585, HALF_WIDTH_BODY_MIN_US = 0.69, BODY_192 = 0.80, BODY_192_MIN_US = 0.88;
+double body_us_for(double active, int tile_n, int dev_cus) {
     const double full_body_us = 1.05 * std::max(1.0, std::pow(active / (0.5 * dev_cus), 0.43));
-    return half_width ? std::max(HALF_WIDTH_BODY_MIN_US, HALF_WIDTH_BODY * full_body_us) : full_body_us;
+    if (tile_n == 128) return std::max(HALF_WIDTH_BODY_MIN_US, HALF_WIDTH_BODY * full_body_us);
+    if (tile_n == 192) return std::max(BODY_192_MIN_US, BODY_192 * full_body_us);
+    return full_body_us;
 }
 // one round of `active` work items of `bodies` loop bodies each, with the store burst that ends it
-double round_us_for(double active, double bodies, bool half_width, int dev_cus) {
-    const double store_us = active * (half_width ? 128.0 : 256.0) * 1024.0 / 4.6e6;
-    return bodies * body_us_for(active, half_width, dev_cus) + store_us + 3.0;
+double round_us_for(double active, double bodies, int tile_n, int dev_cus) {
+    const double store_us = active * (double)tile_n * 1024.0 / 4.6e6;
+    return bodies * body_us_for(active, tile_n, dev_cus) + store_us + 3.0;
 }
 // what adding the slices costs: inside the kernel (every wave stores the rows it does not own, waits for its S - 1
 // partners and reads what they stored for its rows; measured on config-4-like shapes: about 6 us and 12 us per further
 // slice, most of it the wait for the slowest partner - two slices of 128 tiles: 18 us against 22 for the pass; four of 64
 // tiles: 42 against 19; eight of 32 half-width tiles: 44 against 10), or by the reduction pass
-double fused_reduction_us(int S, bool half_width) { return 6.0 + (half_width ? 6.0 : 12.0) * (double)(S - 1); }
+double fused_reduction_us(int S, int tile_n) { return 6.0 + 12.0 * tile_n / 256.0 * (double)(S - 1); }
 double reduction_pass_us(int S, int64_t mn) { return 3.0 + (double)(S + 1) * (double)mn * 4.0 / 5.3e6; }
-double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus, bool half_width, bool fused, int dev_cus) {
+double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus, int tile_n, bool fused, int dev_cus) {
     const double items = (double)tiles * S;
     const double rounds = std::ceil(items / num_cus);
     const double active = items / rounds;   // workgroups (CUs) busy in a round
     const double bodies = (double)K / S / ck::STREAM_K_MULTIPLE_HOST;
-    double t = rounds * round_us_for(active, bodies, half_width, dev_cus);
-    if (S > 1) t += fused ? fused_reduction_us(S, half_width) : reduction_pass_us(S, mn);
+    double t = rounds * round_us_for(active, bodies, tile_n, dev_cus);
+    if (S > 1) t += fused ? fused_reduction_us(S, tile_n) : reduction_pass_us(S, mn);
     return t;
 }
 
 // How the straight-line kernel runs an M x N x K product on num_cus workgroups.
 struct StreamPlan {
-    bool half_width;       // 256 x 128 tiles
+    int tile_n;            // tile width: 256, 192 or 128 columns of D
     int64_t tiles;         // tiles of that width
     int64_t whole_tiles;   // tile counts [0, whole_tiles) run over all of K ...
     int slices;            // ... the others in this many K slices each (1: none are cut, whole_tiles == tiles)
@@ -314,16 +317,16 @@ bool slices_legal(int K, int c) { return c >= 2 && K % (c * ck::STREAM_K_MULTIPL
 // The slices are added inside the kernel where that is allowed - the option; the waves that hold the slices of a wave tile
 // wait for one another, so all of them must be running at once: every workgroup at most one sliced item (sliced_items <=
 // num_cus) and no more workgroups than the device has CUs - and estimated cheaper than the reduction pass.
-bool reduces_in_kernel(const Options& opt, int slices, int64_t sliced_tiles, int64_t mn, int num_cus, bool half_width, int dev_cus) {
+bool reduces_in_kernel(const Options& opt, int slices, int64_t sliced_tiles, int64_t mn, int num_cus, int tile_n, int dev_cus) {
     if (!opt[OPT_FUSED_REDUCTION] || slices < 2 || num_cus > dev_cus || sliced_tiles * slices > num_cus) return false;
-    return opt[OPT_FUSED_REDUCTION] == 2 || fused_reduction_us(slices, half_width) < reduction_pass_us(slices, mn);
+    return opt[OPT_FUSED_REDUCTION] == 2 || fused_reduction_us(slices, tile_n) < reduction_pass_us(slices, mn);
 }
 
 // Number of K slices for `tiles` tiles that all are cut (1: no split). policy 0: never; 1: automatic - with fewer tiles
 // than CUs, the legal slice count whose estimated duration is shortest (a larger count must win by 3 %: it costs scratch
 // memory); >= 2: that many slices if legal, else the next smaller legal count.
 // Legal: slices of whole loop bodies and at least SPLIT_K_MIN_SLICE deep (any tile count, any N).
-int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, const Options& opt, bool half_width, int dev_cus) {
+int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, const Options& opt, int tile_n, int dev_cus) {
     const int policy = opt[OPT_SPLIT_K];
     if (policy == 0 || tiles <= 0) return 1;
     if (policy >= 2) {
@@ -333,10 +336,10 @@ int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, const Options&
     }
     if (tiles >= num_cus) return 1;
     int best = 1;
-    double best_us = split_k_estimate_us(tiles, mn, K, 1, num_cus, half_width, false, dev_cus);
+    double best_us = split_k_estimate_us(tiles, mn, K, 1, num_cus, tile_n, false, dev_cus);
     for (int c = 2; c <= 16; ++c) {
         if (!slices_legal(K, c)) continue;
-        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus, half_width, reduces_in_kernel(opt, c, tiles, mn, num_cus, half_width, dev_cus), dev_cus);
+        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus, tile_n, reduces_in_kernel(opt, c, tiles, mn, num_cus, tile_n, dev_cus), dev_cus);
         if (us < 0.97 * best_us) { best = c; best_us = us; }
     }
     return best;
@@ -360,35 +363,35 @@ int persistent_grid(int64_t tiles, int num_cus, int num_xcd, bool even_rounds) {
 // the full rounds run whole tiles on all num_cus workgroups and the tiles of the partly filled last round are cut into 2
 // to 4 slices reduced in the kernel, in the same launch, where that is estimated at least 5 % shorter than rounds of
 // whole tiles (6144^3 measures the same either way, 391 us: 576 tiles as 2 x 256 whole tiles + 64 tiles in 2 slices, or as
-// 3 rounds of 192 whole tiles; with the 5 % margin it takes the rounds). 256 x 128 tiles where they are
-// estimated at least 5 % faster than 256 x 256 (they fill a device that few large tiles leave idle, at a lower rate per
-// CU), or always / never by the option.
+// 3 rounds of 192 whole tiles; with the 5 % margin it takes the rounds). 256 x 192 or 256 x 128 tiles where they are
+// estimated at least 5 % faster than 256 x 256 (they fill a device that the large tiles leave partly idle, at a lower rate
+// per CU), or always / never by the option.
 StreamPlan stream_plan(int M, int N, int K, int num_cus, const Options& opt) {
     const int64_t mn = (int64_t)M * N;
     const int width = opt[OPT_HALF_WIDTH], dev_cus = device_cus();
     const bool even = opt[OPT_EVEN_ROUNDS] != 0;
-    auto plan = [&](bool half) {
-        const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + (half ? 127 : 255)) / (half ? 128 : 256));
-        StreamPlan p{half, tiles, tiles, 1, false, persistent_grid(tiles, num_cus, opt[OPT_NUM_XCD], even), 0.0};
+    auto plan = [&](int tile_n) {
+        const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + tile_n - 1) / tile_n);
+        StreamPlan p{tile_n, tiles, tiles, 1, false, persistent_grid(tiles, num_cus, opt[OPT_NUM_XCD], even), 0.0};
         if (tiles <= num_cus) {
-            p.slices = split_k_slices(tiles, mn, K, num_cus, opt, half, dev_cus);
-            p.fused = reduces_in_kernel(opt, p.slices, tiles, mn, num_cus, half, dev_cus);
+            p.slices = split_k_slices(tiles, mn, K, num_cus, opt, tile_n, dev_cus);
+            p.fused = reduces_in_kernel(opt, p.slices, tiles, mn, num_cus, tile_n, dev_cus);
             if (p.slices > 1) {
                 p.whole_tiles = 0;
                 p.grid = (int)std::min<int64_t>(tiles * p.slices, num_cus);
             }
-            p.us = split_k_estimate_us(tiles, mn, K, p.slices, num_cus, half, p.fused, dev_cus);
+            p.us = split_k_estimate_us(tiles, mn, K, p.slices, num_cus, tile_n, p.fused, dev_cus);
             return p;
         }
         // rounds of whole tiles (as many rounds as num_cus workgroups need, evenly filled)
         const double rounds = std::ceil((double)tiles / num_cus), bodies = (double)K / ck::STREAM_K_MULTIPLE_HOST;
-        p.us = rounds * round_us_for(even ? (double)tiles / rounds : (double)num_cus, bodies, half, dev_cus);
+        p.us = rounds * round_us_for(even ? (double)tiles / rounds : (double)num_cus, bodies, tile_n, dev_cus);
         const int64_t full = tiles / num_cus * num_cus, rest = tiles - full;
         if (rest > 0 && opt[OPT_TAIL_ROUND] && opt[OPT_FUSED_REDUCTION] && opt[OPT_SPLIT_K] == 1 && num_cus <= dev_cus) {
-            const double head_us = (double)(full / num_cus) * round_us_for(num_cus, bodies, half, dev_cus);
+            const double head_us = (double)(full / num_cus) * round_us_for(num_cus, bodies, tile_n, dev_cus);
             for (int c = 2; c <= TAIL_ROUND_MAX_SLICES; ++c) {
                 if (!slices_legal(K, c) || rest * c > num_cus) continue;
-                const double us = head_us + split_k_estimate_us(rest, mn, K, c, num_cus, half, true, dev_cus);
+                const double us = head_us + split_k_estimate_us(rest, mn, K, c, num_cus, tile_n, true, dev_cus);
                 if (us < 0.95 * p.us) {
                     p.us = us; p.slices = c; p.fused = true; p.whole_tiles = full; p.grid = num_cus;
                 }
@@ -396,11 +399,18 @@ StreamPlan stream_plan(int M, int N, int K, int num_cus, const Options& opt) {
         }
         return p;
     };
-    const StreamPlan full = plan(false);
-    if (width == 0) return full;
-    const StreamPlan half = plan(true);
-    if (width == 2) return half;
-    return half.us < 0.95 * full.us ? half : full;
+    // width option: 0 only 256 x 256 tiles; 1 the width estimated shortest (a narrower one must beat 256 x 256 by 5 %: per CU
+    // it runs at a lower rate, and the estimate is coarse); 2 always 256 x 128; 3 always 256 x 192
+    if (width == 2) return plan(128);
+    if (width == 3) return plan(192);
+    StreamPlan best = plan(256);
+    if (width == 0) return best;
+    const double bar = 0.95 * best.us;
+    for (int tile_n : {192, 128}) {
+        const StreamPlan p = plan(tile_n);
+        if (p.us < bar && p.us < best.us) best = p;
+    }
+    return best;
 }
 
 // Scratch memory of the K slices of a plan. Reduced in the kernel: per sliced tile slices - 1 tiles of fp32 in the
@@ -409,7 +419,7 @@ StreamPlan stream_plan(int M, int N, int K, int num_cus, const Options& opt) {
 constexpr size_t FIX_STATE_BYTES_PER_TILE = 8 * 128;   // eight waves, one counter per 128-byte line (FIX_STATE_STRIDE_BYTES of the kernel)
 size_t fix_state_bytes(const StreamPlan& p) { return (size_t)(p.tiles - p.whole_tiles) * FIX_STATE_BYTES_PER_TILE; }
 size_t fix_partial_bytes(const StreamPlan& p) {
-    return (size_t)(p.tiles - p.whole_tiles) * (size_t)(p.slices - 1) * 256 * (p.half_width ? 128 : 256) * sizeof(float);
+    return (size_t)(p.tiles - p.whole_tiles) * (size_t)(p.slices - 1) * 256 * p.tile_n * sizeof(float);
 }
 
 // The tuning tuple the straight-line kernel is written for (it also needs K in whole loop bodies of 64).
@@ -539,11 +549,11 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         // take 256 x 128 tiles.
         const bool bek = opt[OPT_BARRIER_EVERY_KSTEP] != 0;
         StreamPlan plan = stream_plan(M, N, K, t.num_cus, opt);
-        const bool half = plan.half_width;
-        if (half) a.tiles_n = (N + 127) / 128;
+        const int tile_n = plan.tile_n;
+        a.tiles_n = (N + tile_n - 1) / tile_n;
         const long long count = (long long)M * N;
         auto launch = [&](const GemmArgs& args, int wgs) {
-            return dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(wgs), s, args, bek, half) : launch_gemm_stream_bf16(dim3(wgs), s, args, bek, half);
+            return dtype == CK_DT_F16 ? launch_gemm_stream_f16(dim3(wgs), s, args, bek, tile_n) : launch_gemm_stream_bf16(dim3(wgs), s, args, bek, tile_n);
         };
         // the K slices' scratch memory: a provided buffer that is too small is the caller's error; a failed allocation
         // is not - the launch of whole tiles computes the same product without any
@@ -713,7 +723,7 @@ int ckopt_gemm_launch_plan_ex(int M, int N, int K, int operands_aligned, CK_TUNI
     if (straight_line_tuple(t, opt)) {
         const StreamPlan plan = stream_plan(M, N, launch_k(K, operands_aligned != 0, t, opt), t.num_cus, opt);
         plan_out[0] = 1;
-        plan_out[1] = plan.half_width ? 128 : 256;
+        plan_out[1] = plan.tile_n;
         plan_out[2] = plan.slices;
         plan_out[4] = (int)(plan.tiles - plan.whole_tiles);
         plan_out[5] = plan.slices > 1 && plan.fused ? 1 : 0;

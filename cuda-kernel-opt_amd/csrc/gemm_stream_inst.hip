@@ -8,7 +8,7 @@ static_assert(STREAM_K_MULTIPLE == 64, "the host's slice rule assumes loop bodie
 template <typename DT, bool ODD_ONLY, bool KTAIL, int WTC>
 static hipError_t stream_launch_one(dim3 grid, hipStream_t stream, const GemmArgs& a) {
     auto kern = gemm_stream_kernel<DT, ODD_ONLY, KTAIL, WTC>;
-    constexpr int lds_bytes = stream_lds_bytes(2 * WTC * 16);
+    constexpr int lds_bytes = stream_lds_bytes(2 * WTC * 16);   // (this file holds the 256- and 128-wide instances; gemm_stream_inst_w6.hip the 192-wide ones)
     static bool opted[64] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -27,18 +27,20 @@ template <typename DT, bool ODD_ONLY, int WTC>
 static hipError_t stream_launch_k(dim3 grid, hipStream_t stream, const GemmArgs& a) {
     return a.K % STREAM_K_MULTIPLE == 0 ? stream_launch_one<DT, ODD_ONLY, false, WTC>(grid, stream, a) : stream_launch_one<DT, ODD_ONLY, true, WTC>(grid, stream, a);
 }
+hipError_t launch_gemm_stream_w6(bool bf16, bool odd_only, dim3 grid, hipStream_t stream, const GemmArgs& a);   // gemm_stream_inst_w6.hip
 template <typename DT, bool ODD_ONLY>
-static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a, bool half_width) {
-    return half_width ? stream_launch_k<DT, ODD_ONLY, 4>(grid, stream, a) : stream_launch_k<DT, ODD_ONLY, 8>(grid, stream, a);
+static hipError_t stream_launch(dim3 grid, hipStream_t stream, const GemmArgs& a, int tile_n) {
+    if (tile_n == STREAM_TILE_N_THREE_QUARTERS) return launch_gemm_stream_w6(std::is_same<DT, bf16_tag>::value, ODD_ONLY, grid, stream, a);
+    return tile_n == STREAM_TILE_N_HALF ? stream_launch_k<DT, ODD_ONLY, 4>(grid, stream, a) : stream_launch_k<DT, ODD_ONLY, 8>(grid, stream, a);
 }
 
-// barrier_every_kstep selects the schedule with a barrier in both k-steps of a loop body; half_width the 256 x 128 tiles
-// (a.tiles_n then counts tiles of 128 columns)
-hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, bool half_width) {
-    return barrier_every_kstep ? stream_launch<f16_tag, false>(grid, stream, a, half_width) : stream_launch<f16_tag, true>(grid, stream, a, half_width);
+// barrier_every_kstep selects the schedule with a barrier in both k-steps of a loop body; tile_n the tile width: 256,
+// 192 or 128 columns (a.tiles_n counts tiles of that width)
+hipError_t launch_gemm_stream_f16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, int tile_n) {
+    return barrier_every_kstep ? stream_launch<f16_tag, false>(grid, stream, a, tile_n) : stream_launch<f16_tag, true>(grid, stream, a, tile_n);
 }
-hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, bool half_width) {
-    return barrier_every_kstep ? stream_launch<bf16_tag, false>(grid, stream, a, half_width) : stream_launch<bf16_tag, true>(grid, stream, a, half_width);
+hipError_t launch_gemm_stream_bf16(dim3 grid, hipStream_t stream, const GemmArgs& a, bool barrier_every_kstep, int tile_n) {
+    return barrier_every_kstep ? stream_launch<bf16_tag, false>(grid, stream, a, tile_n) : stream_launch<bf16_tag, true>(grid, stream, a, tile_n);
 }
 
 // what the kernel assumes about a launch (the caller falls back to the general fused kernel otherwise)

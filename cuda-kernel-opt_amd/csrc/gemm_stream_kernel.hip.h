@@ -48,8 +48,12 @@ constexpr int STREAM_SEGK = 32;
 constexpr int STREAM_STAGES = 5;
 constexpr int STREAM_K_MULTIPLE = 2 * STREAM_SEGK;  // one loop body
 constexpr int STREAM_TILE_N_HALF = 128;   // the half-width form: 256 x 128 tiles (wave tiles of 64 x 64)
+constexpr int STREAM_TILE_N_THREE_QUARTERS = 192;   // 256 x 192 tiles (wave tiles of 64 x 96)
 // bytes of the ring for tiles of 256 x tile_n
-constexpr int stream_lds_bytes(int tile_n) { return STREAM_STAGES * (STREAM_TILE + tile_n) * STREAM_SEGK * 2; }
+constexpr int stream_ring_bytes(int tile_n) { return STREAM_STAGES * (STREAM_TILE + tile_n) * STREAM_SEGK * 2; }
+// dynamic LDS of a launch: the ring, and for 256 x 192 tiles 1 KiB behind it that takes the zeros of the loads half of
+// the waves issue only to keep every wave's load count the same
+constexpr int stream_lds_bytes(int tile_n) { return stream_ring_bytes(tile_n) + (tile_n == STREAM_TILE_N_THREE_QUARTERS ? 1024 : 0); }
 constexpr int STREAM_LDS_BYTES = stream_lds_bytes(STREAM_TILE);
 constexpr int FIX_STATE_STRIDE_BYTES = 128;  // bytes between the announcement counters of two (sliced tile, wave) units
 
@@ -59,7 +63,11 @@ constexpr int FIX_STATE_STRIDE_BYTES = 128;  // bytes between the announcement c
 // instructions per load. Launches with K % 64 == 0 run the instance without any of it.
 // WTC: 16-column blocks per wave tile. 8: 256 x 256 tiles (wave tiles of 64 x 128); 4: 256 x 128 tiles (wave tiles of
 // 64 x 64) for launches whose 256 x 256 tiles would leave most of the device idle - twice the tiles, half the MFMAs
-// per k-step and wave, a ring of 24 KiB quarters, one load pair of Bt per wave and body instead of two.
+// per k-step and wave, a ring of 24 KiB quarters, one load pair of Bt per wave and body instead of two; 6: 256 x 192
+// tiles (wave tiles of 64 x 96) for tile counts that fill the last round badly at the other widths (6144^3: 768 tiles
+// = exactly three rounds of 256) - quarters of 28 KiB; Bt's 192 rows are twelve 16-row loads, so waves 0 .. 3 issue a
+// second pair of Bt and waves 4 .. 7 a pair that fetches nothing (every lane out of range, zeros into a spare KiB of
+// LDS): all waves issue the same number of loads, which the counted waits rely on.
 template <typename DT, bool ODD_ONLY, bool KTAIL, int WTC>
 __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     constexpr int TILE = STREAM_TILE, NQ = STREAM_STAGES;
@@ -69,22 +77,26 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     constexpr int OPB = TILE * RB;           // A's part of a quarter
     constexpr int OPB_B = TILE_N * RB;       // Bt's part
     constexpr int QB = OPB + OPB_B;          // one quarter
-    constexpr int B_PAIRS = TILE_N / 128;    // load pairs of Bt per wave and body (16 rows each)
+    constexpr int B_PAIRS = (TILE_N + 127) / 128;   // load pairs of Bt per wave and body (16 rows each; 256 x 192: the second one real in waves 0 .. 3 only)
+    constexpr bool PARTIAL_B3 = TILE_N % 128 != 0;
     constexpr int LPB = (2 + B_PAIRS) * 2;   // loads per wave and body: (A rows w, w + 8; Bt rows w [, w + 8]) x (two halves)
     constexpr int EVEN_LOADS = 4;            // of those, issued in the even k-step when every k-step has a barrier: A's
-    static_assert(WTC == 8 || WTC == 4, "wave tiles of 64 x 128 or 64 x 64");
+    static_assert(WTC == 8 || WTC == 6 || WTC == 4, "wave tiles of 64 x 128, 64 x 96 or 64 x 64");
     // Stores one wave issues in the epilogue of an interior tile. The landing wait of the body behind an epilogue
     // counts them (they sit between the loads in flight and the new ones), so the loops below and the wait
     // immediates are written in terms of the same constants.
     constexpr int F32_GROUP = 2, H16_GROUP = 4;     // accumulator blocks exchanged between lanes into whole lines
     constexpr int STORES_PER_GROUP = 2;             // rows 0..7 and 8..15 of the group
     constexpr int EPILOGUE_STORES = WTR * (WTC / F32_GROUP) * STORES_PER_GROUP;        // fp32 output
-    constexpr int EPILOGUE_STORES_16 = WTR * (WTC / H16_GROUP) * STORES_PER_GROUP;     // 16-bit output
-    static_assert(WTC % F32_GROUP == 0 && WTC % H16_GROUP == 0, "whole groups per wave-tile row");
+    // 16-bit output in whole lines needs groups of four blocks; a wave tile of six block columns (256 x 192 tiles) writes
+    // 16-bit output block by block instead, WTR * WTC = EPILOGUE_STORES stores, and its landing wait counts those
+    constexpr bool H16_WHOLE_LINES = WTC % H16_GROUP == 0;
+    constexpr int EPILOGUE_STORES_16 = H16_WHOLE_LINES ? WTR * (WTC / H16_GROUP) * STORES_PER_GROUP : EPILOGUE_STORES / 2;     // 16-bit output
+    static_assert(WTC % F32_GROUP == 0, "whole groups per wave-tile row");
     static_assert(EPILOGUE_STORES_16 * 2 == EPILOGUE_STORES, "count_stores selects between the two with a shift by one");
     constexpr int PRE = 1;               // columns of MFMAs in front of the barrier
-    constexpr int LOAD_COL_0 = WTC == 8 ? 3 : 1;  // columns behind which a k-step's two load pairs are issued
-    constexpr int LOAD_COL_1 = WTC == 8 ? 6 : 3;
+    constexpr int LOAD_COL_0 = WTC == 8 ? 3 : WTC == 6 ? 2 : 1;  // columns behind which a k-step's two load pairs are issued
+    constexpr int LOAD_COL_1 = WTC == 8 ? 6 : WTC == 6 ? 4 : 3;
     constexpr int FPC = (WTR + WTC + (WTC - PRE) - 1) / (WTC - PRE);   // fragments of the next k-step fetched per column
     static_assert(PRE >= 1 && (WTC - PRE) * FPC >= WTR + WTC && LOAD_COL_0 >= PRE && LOAD_COL_1 > LOAD_COL_0 && LOAD_COL_1 < WTC, "schedule");
     static_assert(LPB + EPILOGUE_STORES < 64 && EPILOGUE_STORES_16 < EPILOGUE_STORES, "the wait immediates must fit the 6-bit counter");
@@ -92,7 +104,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     // store per accumulator block, while the landing wait behind it counts EPILOGUE_STORES: an epilogue that issues fewer
     // stores than the wait counts would let fragments be read before their loads have landed
     static_assert(WTR * WTC >= EPILOGUE_STORES, "the per-block epilogue issues at least the stores the landing wait counts");
-    static_assert(NQ * QB == stream_lds_bytes(TILE_N) && NQ * QB <= LDS_BYTES_PER_CU, "the ring (all of the LDS for 256 x 256 tiles)");
+    static_assert(NQ * QB == stream_ring_bytes(TILE_N) && stream_lds_bytes(TILE_N) <= LDS_BYTES_PER_CU, "the ring (all of the LDS for 256 x 256 tiles)");
 
     extern __shared__ __attribute__((aligned(1024))) char ck_smem[];
     const uint32_t ring_base = (uint32_t)(uintptr_t)(CK_LDS char*)ck_smem;
@@ -153,6 +165,12 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
             toff_hi[h] = absent ? 0x7fffff00u : loff_hi;
         }
     }
+    // 256 x 192 tiles: pair 3 (Bt rows 128 + 16w ..) exists in waves 0 .. 3; in the others every lane's offset lies outside
+    // any descriptor (nothing is fetched) and the zeros go to the spare KiB behind the ring
+    const bool b3_absent = PARTIAL_B3 && wave >= 4;
+    const uint32_t loff_b3 = b3_absent ? 0x7fffff00u : loff_hi;
+    const uint32_t toff_b3[2] = {b3_absent ? 0x7fffff00u : toff_hi[0], b3_absent ? 0x7fffff00u : toff_hi[1]};
+    const uint32_t spare_lds = ring_base + (uint32_t)(NQ * QB);
     uint32_t l_tail = 0;  // KTAIL: nonzero while the body being loaded is the one that holds the end of K
     if constexpr (KTAIL) asm volatile("s_mov_b32 %0, %1" : "=s"(l_tail) : "s"(__builtin_amdgcn_readfirstlane((uint32_t)(kslice <= STREAM_K_MULTIPLE))));
     uint32_t l_kbytes = kwhole_bytes;  // extent along K, in bytes, of the item being loaded
@@ -196,7 +214,16 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         constexpr int HI = P % 2;
         if constexpr (P == 3 && B_PAIRS < 2) return;
         const uint32_t dst = dst_w + (uint32_t)((IS_A ? 0 : OPB) + HI * 8 * 1024);
-        if constexpr (KTAIL) {
+        if constexpr (P == 3 && PARTIAL_B3) {
+            const uint32_t d_lo = b3_absent ? spare_lds : dst + q_lo, d_hi = b3_absent ? spare_lds : dst + q_hi;
+            if constexpr (KTAIL) {
+                dma_load_b128_select(rsrc_b, d_lo, loff_b3, toff_b3[0], l_koff, l_tail);
+                dma_load_b128_select(rsrc_b, d_hi, loff_b3, toff_b3[1], l_koff + (uint32_t)(STREAM_SEGK * 2), l_tail);
+            } else {
+                dma_load_b128(rsrc_b, d_lo, loff_b3, l_koff);
+                dma_load_b128(rsrc_b, d_hi, loff_b3, l_koff + (uint32_t)(STREAM_SEGK * 2));
+            }
+        } else if constexpr (KTAIL) {
             dma_load_b128_select(IS_A ? rsrc_a : rsrc_b, dst + q_lo, HI ? loff_hi : loff_lo, HI ? toff_hi[0] : toff_lo[0], l_koff, l_tail);
             dma_load_b128_select(IS_A ? rsrc_a : rsrc_b, dst + q_hi, HI ? loff_hi : loff_lo, HI ? toff_hi[1] : toff_lo[1],
                                  l_koff + (uint32_t)(STREAM_SEGK * 2), l_tail);
@@ -226,7 +253,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
     // needs D and its rows on 16-byte boundaries). Worked out on the scalar unit in asm: a flag the compiler
     // derives from a compare ends up in a vector register, which the "s" operands of the asm statements
     // below cannot take.
-    const uint32_t d16_misaligned = ((uint32_t)(uintptr_t)g.D | ((uint32_t)g.N << 1)) & 15u;
+    const uint32_t d16_misaligned = H16_WHOLE_LINES ? ((uint32_t)(uintptr_t)g.D | ((uint32_t)g.N << 1)) & 15u : 1u;
     uint32_t count_stores, count_tmp;
     asm volatile("s_lshl_b32 %0, %2, 1\n\ts_cmp_eq_u32 %0, 0\n\ts_cselect_b32 %0, 2, 0\n\t"
                  "s_cmp_eq_u32 %4, 0\n\ts_cselect_b32 %1, %3, 0\n\ts_lshr_b32 %0, %0, %1"
@@ -285,6 +312,12 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                     if (j == 4) issue_pair(std::integral_constant<int, 1>{}, q4, q0);
                     if (j == 6) issue_pair(std::integral_constant<int, 2>{}, q4, q0);
                     if (j == 7) issue_pair(std::integral_constant<int, 3>{}, q4, q0);
+                }
+                if constexpr (P == 1 && WTC == 6) {
+                    if (j == 1) issue_pair(std::integral_constant<int, 0>{}, q4, q0);
+                    if (j == 2) issue_pair(std::integral_constant<int, 1>{}, q4, q0);
+                    if (j == 4) issue_pair(std::integral_constant<int, 2>{}, q4, q0);
+                    if (j == 5) issue_pair(std::integral_constant<int, 3>{}, q4, q0);
                 }
                 if constexpr (P == 1 && WTC == 4) {
                     if (j == 1) issue_pair(std::integral_constant<int, 0>{}, q4, q0);
@@ -482,7 +515,8 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                         if (st + C_DEPTH < EPILOGUE_STORES) cv[st % C_DEPTH] = fetch(st + C_DEPTH);
                     }
                 }
-            } else if (interior && g.out16 && d16_misaligned == 0) {
+            } else if (H16_WHOLE_LINES && interior && g.out16 && d16_misaligned == 0) {
+                if constexpr (H16_WHOLE_LINES) {
                 // 16-bit output in whole 128-byte lines, 16 bytes per lane. A lane's 4 results of a block are
                 // 8 bytes, so two neighbouring blocks swap their odd and even 16-lane rows
                 // (v_permlane16_swap): lane group G = lane / 16 then holds the 8 columns 8 (G / 2) .. of block
@@ -553,6 +587,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                             else *(u32x4*)(d16 + off) = o;
                         }
                     }
+                }
                 }
             } else {
 #pragma unroll

@@ -279,10 +279,12 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  *        start anywhere make every 128-byte run of a row straddle two lines, and only ordinary stores let the parts
  *        meet in L2 before they reach memory (bf16 6143 x 4097 x 3072: 138 us against 164). 1: always non-temporal;
  *        2: never.
- * key 11: tile width of the straight-line kernel. 1 (default): 256 x 128 tiles (wave tiles of 64 x 64, twice the tiles,
- *        0.86 of the rate on a full device) where the launcher's cost model gives them at least 5 % less time than
- *        256 x 256 tiles - tile counts that leave much of the device idle (2560^3: 100 tiles, 53 us -> 37 us);
- *        0: never; 2: always. tile_dim stays 256 in the launcher's parameters.
+ * key 11: tile width of the straight-line kernel. 1 (default): 256 x 192 tiles (wave tiles of 64 x 96, 0.88 of the rate of
+ *        256 x 256 tiles on a full device) or 256 x 128 tiles (wave tiles of 64 x 64, 0.86) where the launcher's cost model
+ *        gives them at least 5 % less time than 256 x 256 tiles - tile counts that fill the last round badly or leave
+ *        much of the device idle (6144^3: 576 tiles in 2.25 rounds -> 768 tiles of 256 x 192 in exactly 3, 395 us ->
+ *        362 us; 3072^3: 65 us -> 57 us; 2560^3: 100 tiles, 53 us -> 37 us with 200 tiles of 256 x 128);
+ *        0: always 256 x 256; 2: always 256 x 128; 3: always 256 x 192. tile_dim stays 256 in the launcher's parameters.
  * key 12: the partly filled last round of the straight-line kernel (default 1). With more tiles than num_sms the last
  *        round leaves CUs idle (6144^3: 576 tiles = 2 x 256 + 64); with 1 its tiles are cut into 2 to 4 K slices that
  *        run as work items of the same launch behind the whole tiles, where the cost model gives that at least 3 % less

@@ -846,7 +846,8 @@ def test_slices_reduced_in_the_kernel_exact(ck, M, N, K, cus, opts):
     prod = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float64)
     da, db, dc = G.to_dev(a), G.to_dev(bt), G.to_dev(c)
     dc16 = G.to_dev(c.astype(np.float16))
-    o = ck.launch_options(fused_reduction=2, **opts)   # 2: in the kernel wherever that is possible, whatever the cost model says
+    # fused_reduction 2: in the kernel wherever that is possible, whatever the cost model says; 256 x 256 tiles unless the case says otherwise
+    o = ck.launch_options(fused_reduction=2, **dict(dict(half_width=0), **opts))
     plan = ck.gemm_launch_plan(M, N, K, True, *tup, options=o)
     if opts.get("tail_round", 1):
         assert plan["sliced_tiles"] > 0 and plan["reduced_in_kernel"], plan
@@ -944,6 +945,71 @@ def test_two_host_threads_with_different_options(ck):
     threads[2].join()
     assert not errors, errors
     assert ck.device_status() == 0
+
+
+@pytest.mark.parametrize("M,N,K,cus,opts,dt_name,out16,beta", [
+    (256, 192, 64, 256, {}, "f16", False, 0.0),                      # one tile, one loop body
+    (512, 768, 1024, 256, {}, "f16", False, 1.0),
+    (700, 500, 1000, 256, {}, "f16", False, 0.0),                    # ragged in M and N, K % 64 != 0: the instance that masks the end of K
+    (700, 500, 1001, 256, {}, "bf16", False, 0.0),                   # K % 8 != 0: zero-padded copies
+    (1024, 1920, 512, 8, {}, "f16", False, 0.0),                     # 40 tiles on 8 workgroups
+    (1024, 1920, 512, 8, dict(barrier_every_kstep=0), "f16", False, -1.0),
+    (700, 500, 1000, 256, dict(barrier_every_kstep=0), "bf16", False, 0.0),
+    (512, 776, 256, 256, {}, "f16", True, 0.0),                      # 16-bit C / D: block by block (no groups of four block columns)
+    (512, 776, 256, 256, {}, "f16", True, 1.0),
+    (512, 772, 256, 256, {}, "bf16", True, -1.0),
+    (512, 768, 8192, 256, dict(split_k=4, fused_reduction=0), "f16", False, 0.0),     # K slices, second pass
+    (512, 768, 8192, 256, dict(split_k=4, fused_reduction=2), "f16", False, 1.0),     # K slices, added in the kernel
+    (512, 768, 6144, 256, dict(split_k=3, fused_reduction=2), "f16", True, 1.0),
+    (1024, 1920, 8192, 16, dict(fused_reduction=2), "f16", False, 0.0),               # partly filled last round at this width
+])
+def test_three_quarter_width_tiles_exact(ck, M, N, K, cus, opts, dt_name, out16, beta):
+    """256 x 192 tiles of the straight-line kernel (wave tiles of 64 x 96), forced: half of the waves issue a load pair that
+    fetches nothing, the 16-bit epilogue goes block by block; every path exact on small integers, every element written."""
+    dt = ck.DT_F16 if dt_name == "f16" else ck.DT_BF16
+    t = _straight_line_tuning(ck, cus)
+    tup = tuple(t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
+                               "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms"))
+    o = ck.launch_options(half_width=3, **opts)
+    plan = ck.gemm_launch_plan(M, N, K, K % 8 == 0, *tup, options=o)
+    assert plan["tile_cols"] == 192, plan
+    a = ck.fill_int(dt, (M, K), 103, 0, -2, 2)
+    bt = ck.fill_int(dt, (N, K), 103, 1, -2, 2)
+    c = ck.fill_int(ck.DT_F32, (M, N), 103, 2, -3, 3)
+    prod = G.as_f64(dt == ck.DT_BF16, a) @ G.as_f64(dt == ck.DT_BF16, bt).T
+    da, db = G.to_dev(a), G.to_dev(bt)
+    if out16:
+        tdt = torch.float16 if dt == ck.DT_F16 else torch.bfloat16
+        dc = torch.from_numpy(c).to(tdt).cuda() if beta else None
+        d = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+        ck.gemm_shmem_tc_async_opt_port_ex(dt, dt, da, db, dc, d, 1.0, beta, M, N, K, *tup, options=o)
+        got = d.float().cpu().numpy()
+        want = torch.from_numpy(prod + beta * c).to(tdt).float().numpy()
+    else:
+        dc = G.to_dev(c) if beta else None
+        d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+        ck.gemm_shmem_tc_async_opt_port_ex(dt, ck.DT_F32, da, db, dc, d, 1.0, beta, M, N, K, *tup, options=o)
+        got = d.cpu().numpy()
+        want = (prod + beta * c).astype(np.float32)
+    assert ck.device_status() == 0
+    assert np.array_equal(got, want), plan
+
+
+def test_three_quarter_width_tiles_chosen_and_within_tolerance(ck, oracle):
+    """3072^3 (144 tiles of 256 x 256: 0.56 of a round): the launcher takes 192 tiles of 256 x 192; random fp16 data against the
+    oracle over sampled rows of every tile row."""
+    M = N = K = 3072
+    t = suggested_tuning(ck, M, N, K)
+    order = [t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
+                            "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms")]
+    assert ck.gemm_launch_plan(M, N, K, True, *order)["tile_cols"] == 192
+    a = ck.fill_uniform(ck.DT_F16, (M, K), 105, 0, -1.0, 1.0)
+    bt = ck.fill_uniform(ck.DT_F16, (N, K), 105, 1, -1.0, 1.0)
+    got = G.run_gemm(ck, ck.DT_F16, a, bt, t=t)
+    assert not np.isnan(got).any()
+    for r0 in list(range(0, M, 256)) + [M - 4]:
+        ref = oracle.gemm(oracle.DT_F16, a, bt, rows=(r0, r0 + 4))
+        assert_close(oracle, ref, got[r0:r0 + 4])
 
 
 @pytest.mark.parametrize("M,N,K", [(512, 512, 256), (700, 390, 1024), (1024, 768, 4096), (260, 1000, 200)])

@@ -231,7 +231,7 @@ def test_normal_and_int_generators(ck):
 
 def test_option_keys_reject_values_outside_their_range(ck):
     # process-wide switches: a bad value changes nothing and reports the error
-    for key, bad in ((ck.OPT_NUM_XCD, 0), (ck.OPT_PRIO_MODE, 3), (ck.OPT_PRODUCER_NAP, -1), (ck.OPT_SPLIT_K, 17), (ck.OPT_D_STORE_POLICY, 3), (ck.OPT_HALF_WIDTH, 3), (99, 1),
+    for key, bad in ((ck.OPT_NUM_XCD, 0), (ck.OPT_PRIO_MODE, 3), (ck.OPT_PRODUCER_NAP, -1), (ck.OPT_SPLIT_K, 17), (ck.OPT_D_STORE_POLICY, 3), (ck.OPT_HALF_WIDTH, 4), (99, 1),
                      (15, 1), (-1, 0), (ck.OPT_SPIN_LIMIT, 0)):
         with pytest.raises(ck.CkoptError):
             ck.set_option(key, bad)
@@ -377,15 +377,21 @@ def test_launch_plan_reports_what_a_launch_will_run(ck):
     # the partly filled last round: 20 tiles on 16 workgroups with a deep K -> 16 whole tiles, then 4 tiles in K slices
     # added inside the kernel, all in one launch of 16 workgroups; switched off: 2 rounds of 10
     tail = (256, 32, 0, 0, 256, 256, 4, 5, 0, 8, 16)
-    p = plan(1024, 1280, 8192, True, *tail)
+    p = plan(1024, 1280, 8192, True, *tail, options=ck.launch_options(half_width=0))
     assert p["sliced_tiles"] == 4 and p["k_slices"] in (2, 3, 4) and p["reduced_in_kernel"] and p["grid"] == 16
     p = plan(1024, 1280, 8192, True, *tail, options=ck.launch_options(tail_round=0))
-    assert p["sliced_tiles"] == 0 and p["k_slices"] == 1 and p["grid"] == 16 and p["tile_cols"] == 256
+    assert p["sliced_tiles"] == 0 and p["k_slices"] == 1 and p["grid"] <= 16 and p["tile_cols"] in (256, 192)
     prev = ck.set_option(ck.OPT_HALF_WIDTH, 0)
     try:
         assert ck.gemm_launch_plan(2560, 2560, 2560, True, *straight)["tile_cols"] == 256
     finally:
         ck.set_option(ck.OPT_HALF_WIDTH, prev)
+    # 256 x 192 tiles where the other widths fill the last round badly: 6144^3 is 576 tiles of 256 x 256 (2.25 rounds) but 768 of
+    # 256 x 192 (exactly 3); 3072^3 is 144 of 256 (0.56 of a round) but 192 of 192 (0.75)
+    assert plan(6144, 6144, 6144, True, *straight)["tile_cols"] == 192 and plan(6144, 6144, 6144, True, *straight)["grid"] == 256
+    assert plan(3072, 3072, 3072, True, *straight)["tile_cols"] == 192
+    assert plan(3072, 3072, 3072, True, *straight, options=ck.launch_options(half_width=0))["tile_cols"] == 256
+    assert plan(8192, 8192, 8192, True, *straight, options=ck.launch_options(half_width=3))["tile_cols"] == 192
     prev = ck.set_option(ck.OPT_STRAIGHT_LINE, 0)
     try:
         assert ck.gemm_launch_plan(8192, 8192, 8192, True, *straight)["straight_line"] is False

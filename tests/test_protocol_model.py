@@ -487,7 +487,16 @@ class StreamModel:
 SCHEDULES = {"barrier_every_kstep": dict(imm=4, imm_stores=36, odd_only=False), "odd_only": dict(imm=0, imm_stores=32, odd_only=True),
              # 256 x 128 tiles: six loads per body (A's four in the even k-step as before, Bt's two in the odd one), 16 stores per epilogue
              "half_width_barrier_every_kstep": dict(imm=4, imm_stores=20, odd_only=False, bt_pairs=1, stores=16),
-             "half_width_odd_only": dict(imm=0, imm_stores=16, odd_only=True, bt_pairs=1, stores=16)}
+             "half_width_odd_only": dict(imm=0, imm_stores=16, odd_only=True, bt_pairs=1, stores=16),
+             # 256 x 192 tiles: eight loads per body in every wave (the second Bt pair of waves 4 .. 7 fetches nothing but is issued
+             # and completes in order like any other), 24 stores per epilogue
+             "three_quarter_width_barrier_every_kstep": dict(imm=4, imm_stores=28, odd_only=False, bt_pairs=2, stores=24),
+             "three_quarter_width_odd_only": dict(imm=0, imm_stores=24, odd_only=True, bt_pairs=2, stores=24),
+             # an epilogue that issues MORE stores than the landing wait counts is safe (the wait only gets longer): 16-bit output
+             # off the 16-byte boundaries goes through the per-block epilogue (one store per accumulator block, 32) and element-wise
+             # epilogues issue several stores per block, while the wait counts the 32 of the whole-line form
+             "per_block_epilogue": dict(imm=4, imm_stores=36, odd_only=False, stores=32),
+             "element_wise_epilogue": dict(imm=4, imm_stores=36, odd_only=False, stores=64)}
 
 
 @pytest.mark.parametrize("schedule", sorted(SCHEDULES))
@@ -524,6 +533,13 @@ def test_stream_model_detects_wrong_immediates():
             m.run()
             caught += bool(m.errors)
         assert caught > 0
+    # an epilogue that issues FEWER stores than the wait counts (what the kernel's static_assert on the per-block path rules out)
+    caught = 0
+    for seed in range(20):
+        m = StreamModel(8, 1, 6, random.Random(seed), imm=4, imm_stores=36, completion_rate=0.3, slow_wave=seed % 8, stores=16)
+        m.run()
+        caught += bool(m.errors)
+    assert caught > 0
     # 256 x 128 tiles (16 stores per epilogue): one store too many allowed in flight, and the full-width immediate
     for imm_stores in (21, 36):
         caught = 0
