@@ -470,7 +470,7 @@ class StreamModel:
         steps = 0
         while alive:
             steps += 1
-            if steps > 2000000:
+            if steps > 8000000:
                 return "deadlock"
             if self.rng.random() < self.completion_rate:
                 self.complete_some()
@@ -496,7 +496,7 @@ SCHEDULES = {"barrier_every_kstep": dict(imm=4, imm_stores=36, odd_only=False), 
              # off the 16-byte boundaries goes through the per-block epilogue (one store per accumulator block, 32) and element-wise
              # epilogues issue several stores per block, while the wait counts the 32 of the whole-line form
              "per_block_epilogue": dict(imm=4, imm_stores=36, odd_only=False, stores=32),
-             "element_wise_epilogue": dict(imm=4, imm_stores=36, odd_only=False, stores=64)}
+             "element_wise_epilogue": dict(imm=4, imm_stores=36, odd_only=False, stores=48)}
 
 
 @pytest.mark.parametrize("schedule", sorted(SCHEDULES))
