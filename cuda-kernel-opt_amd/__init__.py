@@ -85,6 +85,8 @@ _lib.ckopt_matmul_shmem_lds_req.restype = _i
 _lib.ckopt_matmul_shmem_lds_req.argtypes = [_i, _i]
 _lib.ckopt_check_matmul_shmem_tuning.restype = _i
 _lib.ckopt_check_matmul_shmem_tuning.argtypes = [_i, _i]
+_lib.ckopt_trim_scratch_pool.restype = _i
+_lib.ckopt_trim_scratch_pool.argtypes = [ctypes.c_size_t]
 _lib.ckopt_device_status.restype = _i
 _lib.ckopt_device_status.argtypes = [_p]
 _lib.ckopt_last_launch_clocks.restype = _i
@@ -111,7 +113,7 @@ EXPORTED_SYMBOLS = [
     "ckopt_gemm_shmem_tc_async_opt_port_1", "ckopt_gemm_shmem_tc_async_opt_port_1_lp",
     "ckopt_gemm_shmem_tc_async_opt_port_0", "ckopt_gemm_shmem_tc_async_opt_port_0_lp", "ckopt_get_lds_req", "ckopt_get_num_acc", "ckopt_get_warp_tile_rows",
     "ckopt_get_tile_offset_cd", "ckopt_check_gemm_tuning", "ckopt_matmul_shmem", "ckopt_matmul_shmem_lds_req",
-    "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks",
+    "ckopt_check_matmul_shmem_tuning", "ckopt_device_status", "ckopt_last_launch_clocks", "ckopt_trim_scratch_pool",
     "ckopt_suggest_gemm_tuning",
     "ckopt_set_option", "ckopt_fill_uniform",
     "ckopt_fill_normal", "ckopt_fill_int", "ckopt_fill_constant", "ckopt_error_string",
@@ -331,6 +333,11 @@ def matmul_shmem_lds_req(dtype, tile_dim):
 
 def check_matmul_shmem_tuning(tile_dim, block_rows):
     return _lib.ckopt_check_matmul_shmem_tuning(tile_dim, block_rows)
+
+
+def trim_scratch_pool(keep_bytes=0):
+    """Hands back what the library's stream-ordered scratch pool of the current device holds beyond keep_bytes."""
+    _check(_lib.ckopt_trim_scratch_pool(int(keep_bytes)), "trim_scratch_pool")
 
 
 def device_status(stream=None):

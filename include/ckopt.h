@@ -12,7 +12,8 @@
  * Device memory beyond the operands is needed in two cases only (zero-padded operand copies when K % 8 != 0 or an
  * operand is off a 16-byte boundary; partial planes when the straight-line kernel cuts K into slices). The reference's
  * launcher needs none and allocates nothing (port_2.cu:1088-1168; its drivers own all memory, :1200-1203). Here the
- * plain entry points take it from stream-ordered allocations on `stream` (hipMallocAsync / hipFreeAsync);
+ * plain entry points take it from stream-ordered allocations on `stream`, out of a memory pool the library keeps per
+ * device (freed blocks stay in the pool for the next launch; ckopt_trim_scratch_pool hands them back);
  * ckopt_gemm_shmem_tc_async_opt_port_2_ws takes it from a workspace the caller owns and allocates nothing;
  * ckopt_gemm_shmem_tc_async_opt_port_2_noalloc takes it from a static array inside the library.
  */
@@ -234,6 +235,11 @@ int ckopt_matmul_shmem(int dtype, const void* A, const void* B, void* C, int M, 
 /* Role of get_shmem_req<DT>(tile_dim) (matmul_shmem.cu:138-141). */
 int ckopt_matmul_shmem_lds_req(int dtype, int tile_dim);
 int ckopt_check_matmul_shmem_tuning(int tile_dim, int block_rows);
+
+/* Releases what the library's stream-ordered scratch pool of the current device holds beyond keep_bytes (0: everything
+ * that is not in use). The pool keeps the largest scratch a launch of the allocating entry points has used on the device,
+ * so that the next launch does not pay for a fresh allocation. No reference counterpart. */
+int ckopt_trim_scratch_pool(size_t keep_bytes);
 
 /* Waits for `stream`, then returns the device status word of the current device and clears it:
  * 0 = all flag waits inside the GEMM kernels completed; bit 0 / bit 1 = a producer / consumer wave
