@@ -435,6 +435,13 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
         // D = alpha * acc + beta * C for the block rows `own_rows` of this wave's wave tile, straight from the accumulators;
         // returns whether the tile is an interior one (every wave then issues exactly the stores the next body's landing wait counts)
         auto write_tile = [&](int64_t tc, int slice, unsigned own_rows) __attribute__((always_inline)) {
+            // Every value of C fetched ahead of its use passes through here at the point of use, on every path. The
+            // compiler waits for a load where its result is used; when it moves the use under a condition (a row past the
+            // edge, beta == 0), the paths that skip the use leave the load in flight as far as it can tell, all the way
+            // round to the main loop. There it then waits for ALL loads (vmcnt(0): it knows nothing of the ring's, which
+            // are issued from asm) in front of the first LDS read that reuses the register, and the load queue runs
+            // empty once per k-step (measured on 16384^3: 7 % of the launch). The empty asm is a use no path can skip.
+            auto landed = [](auto& x) __attribute__((always_inline)) { asm volatile("" : "+v"(x)); };
             const bool sliced = slice >= 0;
             const TileRC rc = tile_order(g.tiles_m, g.tiles_n, g.tile_group_m, tc);
             GemmArgs go = g;  // without the reduction in the kernel a K slice writes its own plane of the workspace D points at
@@ -510,6 +517,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
                     for (int st = 0; st < EPILOGUE_STORES; ++st) {
                         f32x4 v = exchanged(st / (GROUPS * STORES_PER_GROUP), ((st / STORES_PER_GROUP) % GROUPS) * F32_GROUP, st % STORES_PER_GROUP);
+                        landed(cv[st % C_DEPTH]);
                         v += cv[st % C_DEPTH] * beta;
                         if (row_of(st) < g.M) put(off_of(st), v);
                         if (st + C_DEPTH < EPILOGUE_STORES) cv[st % C_DEPTH] = fetch(st + C_DEPTH);
@@ -569,6 +577,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                     for (int j = 0; j < WTC; j += H16_GROUP) {
                         const int gi = i * GROUPS16 + j / H16_GROUP;   // this group; the next one's C goes into the other buffer
                         if (gi + 1 < WTR * GROUPS16) fetch_c((gi + 1) / GROUPS16, ((gi + 1) % GROUPS16) * H16_GROUP, cq[(gi + 1) % 2]);
+                        landed(cq[gi % 2][0]); landed(cq[gi % 2][1]); landed(cq[gi % 2][2]); landed(cq[gi % 2][3]);
                         if (!(own_rows & (1u << i))) continue;   // a block row another slice's wave writes
                         const u32x4 first = packed_pair(scaled(acc[i][j], cq[gi % 2][0]), scaled(acc[i][j + 1], cq[gi % 2][1]));
                         const u32x4 second = packed_pair(scaled(acc[i][j + 2], cq[gi % 2][2]), scaled(acc[i][j + 3], cq[gi % 2][3]));

@@ -311,6 +311,53 @@ def test_matmul_shmem_multiply_adds_avoid_one_bank_operands(tmp_path):
     assert checked >= 16
 
 
+def test_straight_line_kernel_main_loops_hold_no_wait_of_the_compilers(tmp_path):
+    """The ring's loads are issued from asm, so the compiler does not know of them: a vector-memory wait it inserts
+    into the main loop on its own account (for a load of C it believes in flight on some path out of the epilogue)
+    is a wait for everything (vmcnt(0)), and it empties the load queue once per k-step. The kernel's own waits sit
+    inside asm statements; in the compiled code of the default instances (both element types, the three tile widths,
+    and the K-tail form) no block with MFMAs may hold any other."""
+    import importlib.util
+    import subprocess
+    spec = importlib.util.spec_from_file_location("ckopt_build", os.path.join(ROOT, "cuda-kernel-opt_amd", "build.py"))
+    b = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(b)
+    csrc = os.path.join(ROOT, "cuda-kernel-opt_amd", "csrc")
+    unit = tmp_path / "stream_instances.hip"
+    wanted = [("f16_tag", "false", 8), ("bf16_tag", "false", 8), ("f16_tag", "true", 8), ("bf16_tag", "true", 8),
+              ("f16_tag", "false", 6), ("bf16_tag", "false", 6), ("f16_tag", "false", 4), ("bf16_tag", "false", 4)]
+    unit.write_text('#include "gemm_stream_kernel.hip.h"\nnamespace ck {\n' + "".join(
+        "template __global__ void gemm_stream_kernel<%s, false, %s, %d>(const GemmArgs);\n" % w for w in wanted) + "}\n")
+    out = str(tmp_path / "stream.s")
+    flags = [f for f in b.DEVICE_FLAGS if f != "-fPIC"]
+    r = subprocess.run([b.HIPCC] + flags + ["-I", csrc, "-S", "--cuda-device-only", str(unit), "-o", out], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    kernel, block, in_asm, loops = None, None, False, {}
+    for line in open(out):
+        m = re.match(r"^(_ZN2ck18gemm_stream_kernel\S*):", line)
+        if m:
+            kernel, block = m.group(1), "entry"
+            continue
+        m = re.match(r"^(\.LBB\d+_\d+):", line)
+        if m:
+            block = m.group(1)
+            continue
+        if kernel is None:
+            continue
+        if "#ASMSTART" in line or "#ASMEND" in line:
+            in_asm = "#ASMSTART" in line
+            continue
+        entry = loops.setdefault((kernel, block), [0, []])
+        if "v_mfma" in line:
+            entry[0] += 1
+        if not in_asm and "s_waitcnt" in line and "vmcnt" in line:
+            entry[1].append(line.strip())
+    main_loops = {k: v for k, v in loops.items() if v[0] >= 32}   # one loop body: two k-steps of 16, 24 or 32 MFMAs
+    assert len({k[0] for k in main_loops}) == len(wanted)
+    for (kernel, block), (mfmas, waits) in main_loops.items():
+        assert not waits, "%s %s (%d MFMAs): %s" % (kernel, block, mfmas, waits)
+
+
 def test_workspace_query_follows_the_launcher_rules(ck):
     # pure host arithmetic (no GPU call): what a launch takes from a caller-owned workspace
     straight = (256, 32, 0, 0, 256, 256, 4, 5, 0, 8, 256)
