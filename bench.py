@@ -54,21 +54,22 @@ def load_package():
     return mod
 
 
-def mfma_ceiling(random_operands, with_loads, ksteps=400000):
+def mfma_ceiling(random_operands, with_loads, ksteps=400000, waves=8):
     """TFLOP/s the bare inner loop of the 256 x 256 tile GEMM sustains on the current device (no synchronisation, no
     waiting for data, no epilogue): cuda-kernel-opt_amd/lib/libckmeasure.so, a measurement aid outside the product
-    library. int ckmeasure_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out)."""
+    library. waves: 8 (wave tiles of 64 x 128, the kernels' shape) or 4 (128 x 128, one wave per SIMD).
+    int ckmeasure_mfma_ceiling_shape(int waves, int random_operands, int with_loads, int ksteps, double* tflops_out)."""
     import ctypes
     path = os.path.join(ROOT, "cuda-kernel-opt_amd", "lib", "libckmeasure.so")
     if not os.path.exists(path):
         raise RuntimeError("libckmeasure.so is not built; run `python cuda-kernel-opt_amd/build.py`")
     lib = ctypes.CDLL(path)
-    lib.ckmeasure_mfma_ceiling.restype = ctypes.c_int
-    lib.ckmeasure_mfma_ceiling.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    lib.ckmeasure_mfma_ceiling_shape.restype = ctypes.c_int
+    lib.ckmeasure_mfma_ceiling_shape.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
     out = ctypes.c_double(0.0)
-    rc = lib.ckmeasure_mfma_ceiling(int(bool(random_operands)), int(bool(with_loads)), int(ksteps), ctypes.byref(out))
+    rc = lib.ckmeasure_mfma_ceiling_shape(int(waves), int(bool(random_operands)), int(bool(with_loads)), int(ksteps), ctypes.byref(out))
     if rc != 0:
-        raise RuntimeError("ckmeasure_mfma_ceiling failed (%d)" % rc)
+        raise RuntimeError("ckmeasure_mfma_ceiling_shape failed (%d)" % rc)
     return out.value
 
 
@@ -411,6 +412,8 @@ def main():
             for loads in (0, 1):
                 key = "%s_operands_%s" % ("random" if rnd else "constant", "with_loads" if loads else "no_loads")
                 res[key] = round(mfma_ceiling(rnd, loads, 400000), 1)
+                # the same loop with one wave per SIMD and wave tiles of 128 x 128 (a third fewer LDS bytes per MFMA)
+                res["four_waves_128x128_" + key] = round(mfma_ceiling(rnd, loads, 400000, waves=4), 1)
             res["fp32_valu_%s_operands" % ("random" if rnd else "constant")] = round(valu_ceiling(rnd), 1)
         print(json.dumps({"probe": "bare inner loop of the 256x256 tile GEMM, 8 waves per CU, ~0.2 s per case",
                           "unit": "TFLOP/s", "nominal_peak": PEAK_TFLOPS["mfma_f16"], **res}))

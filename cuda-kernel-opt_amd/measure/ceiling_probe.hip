@@ -6,6 +6,9 @@
 // sustains is the ceiling a kernel of this shape can reach on the device at hand: with constant
 // operand values the matrix cores run near their nominal rate, with random operand values the
 // device's power limit lowers the clock well below it.
+// A second shape of the same loop answers whether bigger wave tiles would pay: four waves per CU (one per SIMD, all
+// 512 registers each) with wave tiles of 128 x 128 - 64 MFMAs on 16 fragment reads per k-step, a third fewer LDS
+// bytes per MFMA than the eight-wave shape's 32 on 12, at the price of one wave per SIMD.
 #include <hip/hip_runtime.h>
 
 #include <stdint.h>
@@ -28,13 +31,19 @@ __device__ __forceinline__ void probe_dma_b128(i32x4 rsrc, uint32_t lds_dst, uin
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" : : "s"(lds_dst), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
-template <bool RANDOM, bool LOADS>
-__global__ __launch_bounds__(512) void ceiling_probe_kernel(const char* window, int ksteps, float* sink) {
+template <int WAVES, bool RANDOM, bool LOADS>
+__global__ __launch_bounds__(WAVES * 64) void ceiling_probe_kernel(const char* window, int ksteps, float* sink) {
+    constexpr int NT = WAVES * 64;
+    constexpr int WTC = 8, WTR = 32 / WAVES;         // 16 x 16 blocks per wave tile: 4 x 8 (eight waves) or 8 x 8 (four)
+    constexpr int NF = WTR + WTC;                    // fragments per k-step
+    constexpr int FPJ = (NF + WTC - 1) / WTC;        // of which fetched per column of MFMAs
+    constexpr int LOADS_PER_KSTEP = 32 / WAVES;      // 1 KiB loads per wave and k-step: 32 KiB per workgroup either way
+    static_assert(WAVES == 8 || WAVES == 4, "two waves per SIMD with 64 x 128 wave tiles, or one with 128 x 128");
     extern __shared__ __attribute__((aligned(1024))) char probe_smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(CKP_LDS char*)probe_smem;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     // the first 64 KiB play the ring stage the fragments come from, the second 64 KiB receive the loads
-    for (int i = threadIdx.x; i < PROBE_LDS_BYTES / 4; i += 512) {
+    for (int i = threadIdx.x; i < PROBE_LDS_BYTES / 4; i += NT) {
         uint32_t v = 0x3c003c00u;  // two fp16 ones
         if (RANDOM) {
             uint32_t h = (uint32_t)i * 2654435761u + blockIdx.x * 40503u;
@@ -53,64 +62,69 @@ __global__ __launch_bounds__(512) void ceiling_probe_kernel(const char* window, 
     // 8 rows x 128 bytes per wave load, rows 16 KiB apart (the pitch of a K = 8192 fp16 operand)
     const uint32_t voff = (uint32_t)(lane / 8) * 16384u + (uint32_t)(lane % 8) * 16u;
     const int lr = lane & 15, lg = lane >> 4, key = (lr >> 1) % 8;
-    const uint32_t a_lane = lds0 + (uint32_t)((wave / 2) * 64 + lr) * 128u + (uint32_t)((lg ^ key) * 16);
+    const uint32_t a_lane = lds0 + (uint32_t)((wave / 2) * WTR * 16 + lr) * 128u + (uint32_t)((lg ^ key) * 16);
     const uint32_t b_lane = lds0 + 32768u + (uint32_t)((wave % 2) * 128 + lr) * 128u + (uint32_t)((lg ^ key) * 16);
-    u32x4 fr[2][12];
+    u32x4 fr[2][NF];
 #pragma unroll
-    for (int i = 0; i < 12; ++i) {
+    for (int i = 0; i < NF; ++i) {
         fr[0][i] = u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
         fr[1][i] = fr[0][i];
     }
-    f32x4 acc[4][8];
+    f32x4 acc[WTR][WTC];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < WTR; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < WTC; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     __syncthreads();
     uint32_t gpos = 0;
     for (int it = 0; it < ksteps; it += 2) {
 #pragma unroll
         for (int P = 0; P < 2; ++P) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < WTC; ++j) {
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const int f = j * 2 + q;
-                    if (f < 4) fr[1 - P][f] = *(const CKP_LDS u32x4*)(uintptr_t)((a_lane ^ (uint32_t)(P * 64)) + f * 2048);
-                    else if (f < 12) fr[1 - P][f] = *(const CKP_LDS u32x4*)(uintptr_t)((b_lane ^ (uint32_t)(P * 64)) + (f - 4) * 2048);
+                for (int q = 0; q < FPJ; ++q) {
+                    const int f = j * FPJ + q;
+                    if (f < WTR) fr[1 - P][f] = *(const CKP_LDS u32x4*)(uintptr_t)((a_lane ^ (uint32_t)(P * 64)) + f * 2048);
+                    else if (f < NF) fr[1 - P][f] = *(const CKP_LDS u32x4*)(uintptr_t)((b_lane ^ (uint32_t)(P * 64)) + (f - WTR) * 2048);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (LOADS && j % 2 == 0) {
+                if (LOADS) {
                     // distinct lines per wave and load; the window (4 row groups x 16 KiB of k) wraps
-                    const int d = j / 2;
-                    probe_dma_b128(rsrc, lds0 + 65536u + (uint32_t)(wave * 4 + d) * 1024u, voff,
-                                   ((gpos + (uint32_t)(wave * 4 + d) * 128u) & 0x3fffu) + ((gpos >> 14) & 3u) * 131072u);
+#pragma unroll
+                    for (int d = j * LOADS_PER_KSTEP / WTC; d < (j + 1) * LOADS_PER_KSTEP / WTC; ++d)
+                        probe_dma_b128(rsrc, lds0 + 65536u + (uint32_t)(wave * LOADS_PER_KSTEP + d) * 1024u, voff,
+                                       ((gpos + (uint32_t)(wave * LOADS_PER_KSTEP + d) * 128u) & 0x3fffu) + ((gpos >> 14) & 3u) * 131072u);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fr[P][4 + j]), __builtin_bit_cast(f16x8, fr[P][i]), acc[i][j], 0, 0, 0);
+                for (int i = 0; i < WTR; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fr[P][WTR + j]), __builtin_bit_cast(f16x8, fr[P][i]), acc[i][j], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (LOADS) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-            gpos += 8u * 4u * 128u;
+            // the loads of the two k-steps before this one may still fly
+            if (LOADS) {
+                if (LOADS_PER_KSTEP == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+            }
+            gpos += 32u * 128u;
         }
     }
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     float s = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < WTR; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) s += acc[i][j][0] + acc[i][j][3];
-    sink[blockIdx.x * 512 + threadIdx.x] = s;
+        for (int j = 0; j < WTC; ++j) s += acc[i][j][0] + acc[i][j][3];
+    sink[blockIdx.x * NT + threadIdx.x] = s;
 }
 
-template <bool RANDOM, bool LOADS>
+template <int WAVES, bool RANDOM, bool LOADS>
 hipError_t launch_probe(int cus, const char* window, int ksteps, float* sink, hipStream_t s) {
-    auto kern = ceiling_probe_kernel<RANDOM, LOADS>;
+    auto kern = ceiling_probe_kernel<WAVES, RANDOM, LOADS>;
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, ck::LDS_BYTES_PER_CU);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(cus), dim3(512), PROBE_LDS_BYTES, s, window, ksteps, sink);
+    hipLaunchKernelGGL(kern, dim3(cus), dim3(WAVES * 64), PROBE_LDS_BYTES, s, window, ksteps, sink);
     return hipGetLastError();
 }
 
@@ -196,10 +210,10 @@ extern "C" int ckmeasure_valu_ceiling(int random_operands, int iters, double* tf
 // Built into lib/libckmeasure.so, a measurement aid that bench.py loads next to the product library (which does not
 // contain it). random_operands: random instead of constant fragment values; with_loads: also the direct-to-LDS loads;
 // runs ksteps k-steps per wave on every CU after a warm-up, allocates and frees its own buffers, synchronises, and
-// returns the rate in TFLOP/s.
-extern "C" int ckmeasure_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out) {
+// returns the rate in TFLOP/s. waves: 8 (wave tiles of 64 x 128, the GEMM kernels' shape) or 4 (128 x 128).
+extern "C" int ckmeasure_mfma_ceiling_shape(int waves, int random_operands, int with_loads, int ksteps, double* tflops_out) {
     using namespace ck;
-    if (!tflops_out || ksteps < 2 || ksteps > (1 << 26)) return CK_ERR_BAD_PARAM;
+    if (!tflops_out || ksteps < 2 || ksteps > (1 << 26) || !(waves == 8 || waves == 4)) return CK_ERR_BAD_PARAM;
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
         return CK_ERR_HIP;
@@ -215,8 +229,12 @@ extern "C" int ckmeasure_mfma_ceiling(int random_operands, int with_loads, int k
         if (hipMemset(window, 0, window_bytes) != hipSuccess) break;
         if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) break;
         auto go = [&](int n) {
-            if (random_operands) return with_loads ? launch_probe<true, true>(cus, window, n, sink, nullptr) : launch_probe<true, false>(cus, window, n, sink, nullptr);
-            return with_loads ? launch_probe<false, true>(cus, window, n, sink, nullptr) : launch_probe<false, false>(cus, window, n, sink, nullptr);
+            if (waves == 4) {
+                if (random_operands) return with_loads ? launch_probe<4, true, true>(cus, window, n, sink, nullptr) : launch_probe<4, true, false>(cus, window, n, sink, nullptr);
+                return with_loads ? launch_probe<4, false, true>(cus, window, n, sink, nullptr) : launch_probe<4, false, false>(cus, window, n, sink, nullptr);
+            }
+            if (random_operands) return with_loads ? launch_probe<8, true, true>(cus, window, n, sink, nullptr) : launch_probe<8, true, false>(cus, window, n, sink, nullptr);
+            return with_loads ? launch_probe<8, false, true>(cus, window, n, sink, nullptr) : launch_probe<8, false, false>(cus, window, n, sink, nullptr);
         };
         if (go(ksteps / 8 + 2) != hipSuccess) break;   // warm-up
         if (hipEventRecord(e0, nullptr) != hipSuccess) break;
@@ -225,8 +243,8 @@ extern "C" int ckmeasure_mfma_ceiling(int random_operands, int with_loads, int k
         float ms = 0.f;
         if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess || ms <= 0.f) break;
         const int n = (ksteps + 1) / 2 * 2;
-        // per CU and k-step: 8 waves x 32 MFMAs x 16*16*32*2 flop = a 256 x 256 x 32 block
-        *tflops_out = (double)cus * n * 8.0 * 32.0 * 16384.0 / (ms * 1e-3) * 1e-12;
+        // per CU and k-step: 256 MFMAs (8 waves x 32 or 4 x 64) x 16*16*32*2 flop = a 256 x 256 x 32 block
+        *tflops_out = (double)cus * n * 256.0 * 16384.0 / (ms * 1e-3) * 1e-12;
         rc = CK_OK;
     } while (false);
     if (e0) (void)hipEventDestroy(e0);
@@ -234,4 +252,8 @@ extern "C" int ckmeasure_mfma_ceiling(int random_operands, int with_loads, int k
     if (window) (void)hipFree(window);
     if (sink) (void)hipFree(sink);
     return rc;
+}
+
+extern "C" int ckmeasure_mfma_ceiling(int random_operands, int with_loads, int ksteps, double* tflops_out) {
+    return ckmeasure_mfma_ceiling_shape(8, random_operands, with_loads, ksteps, tflops_out);
 }
