@@ -316,10 +316,10 @@ double round_us_for(double active, double bodies, int tile_n, int dev_cus) {
     return bodies * body_us_for(active, tile_n, dev_cus) + store_us + 3.0;
 }
 // what adding the slices costs: inside the kernel (every wave stores the rows it does not own, waits for its S - 1
-// partners and reads what they stored for its rows; measured on config-4-like shapes: about 6 us and 12 us per further
-// slice, most of it the wait for the slowest partner - two slices of 128 tiles: 18 us against 22 for the pass; four of 64
-// tiles: 42 against 19; eight of 32 half-width tiles: 44 against 10), or by the reduction pass
-double fused_reduction_us(int S, int tile_n) { return 6.0 + 12.0 * tile_n / 256.0 * (double)(S - 1); }
+// partners and reads what they stored for its rows; most of it is the wait for the slowest partner, which does not shrink
+// with the tile: measured against the pass, two slices of 128 tiles of 256 x 256: 18 us against 22; of 128 tiles of 256 x 128
+// (512 x 8192 x 8192, 256 x 16384 x 4096): 16 against 12; four slices of 64 tiles: 42 against 19), or by the reduction pass
+double fused_reduction_us(int S, int /*tile_n*/) { return 4.0 + 14.0 * (double)(S - 1); }
 double reduction_pass_us(int S, int64_t mn) { return 3.0 + (double)(S + 1) * (double)mn * 4.0 / 5.3e6; }
 double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus, int tile_n, bool fused, int dev_cus) {
     const double items = (double)tiles * S;
