@@ -114,7 +114,13 @@ int ckopt_gemm_shmem_tc_async_opt_port_2_ws(int dtype, int cd_dtype, const void*
  * allocating library routine is called. A launch that needs more than the array holds (both pieces, each rounded up
  * to 256 bytes) returns CKOPT_ERR_TOO_LARGE and D is not written; ckopt_set_option(7, 0) makes such a launch
  * fit by not cutting K. Every device holds one array and every call on a device uses it: calls that overlap on one
- * device (different streams, different threads) race on it. Nothing in it needs to start at zero. */
+ * device (different streams, different threads) race on it. Nothing in it needs to start at zero (the counters of
+ * a reduction inside the kernel are cleared by a small kernel of the same launch, not by a memset).
+ * Before a launch is recorded into a HIP graph, one eager call with the same element type, shape class (K a
+ * multiple of 64 or not, the tile width the plan query reports) and options must have run on the device: the first
+ * call on a device resolves the array's address and the first use of each kernel instance sets its LDS-size
+ * attribute, neither of which may happen under capture. The array is resident on every device the process uses the
+ * library on, whether or not this entry point is ever called. */
 #define CKOPT_NOALLOC_SCRATCH_BYTES (64u << 20)
 int ckopt_gemm_shmem_tc_async_opt_port_2_noalloc(int dtype, const void* A, const void* Bt, const float* C, float* D,
                                                  float alpha, float beta, int M, int N, int K, int tile_dim,
