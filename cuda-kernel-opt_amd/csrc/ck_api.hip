@@ -315,11 +315,11 @@ double round_us_for(double active, double bodies, int tile_n, int dev_cus) {
     const double store_us = active * (double)tile_n * 1024.0 / 4.6e6;
     return bodies * body_us_for(active, tile_n, dev_cus) + store_us + 3.0;
 }
-// what adding the slices costs: inside the kernel (every wave stores the rows it does not own, waits for its S - 1
-// partners and reads what they stored for its rows; most of it is the wait for the slowest partner, which does not shrink
-// with the tile: measured against the pass, two slices of 128 tiles of 256 x 256: 18 us against 22; of 128 tiles of 256 x 128
-// (512 x 8192 x 8192, 256 x 16384 x 4096): 16 against 12; four slices of 64 tiles: 42 against 19), or by the reduction pass
-double fused_reduction_us(int S, int /*tile_n*/) { return 4.0 + 14.0 * (double)(S - 1); }
+// what adding the slices costs: inside the kernel (every wave stores its partial sums and counts itself; the one that
+// comes last reads the other S - 1 partials, a block row of 8 KiB at a time, and writes the tile alone - a chain of
+// memory round trips at the end of the launch, once per sliced item of a workgroup; measured against the pass: two slices
+// of 128 tiles 27 us against 22, three of 81 tiles 35 against 19, four of 64 tiles 47 against 19), or by the reduction pass
+double fused_reduction_us(int S, double sliced_items_per_workgroup) { return (17.0 + 10.0 * (double)(S - 1)) * std::max(1.0, sliced_items_per_workgroup); }
 double reduction_pass_us(int S, int64_t mn) { return 3.0 + (double)(S + 1) * (double)mn * 4.0 / 5.3e6; }
 double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus, int tile_n, bool fused, int dev_cus) {
     const double items = (double)tiles * S;
@@ -327,7 +327,7 @@ double split_k_estimate_us(int64_t tiles, int64_t mn, int K, int S, int num_cus,
     const double active = items / rounds;   // workgroups (CUs) busy in a round
     const double bodies = (double)K / S / ck::STREAM_K_MULTIPLE_HOST;
     double t = rounds * round_us_for(active, bodies, tile_n, dev_cus);
-    if (S > 1) t += fused ? fused_reduction_us(S, tile_n) : reduction_pass_us(S, mn);
+    if (S > 1) t += fused ? fused_reduction_us(S, rounds) : reduction_pass_us(S, mn);
     return t;
 }
 
@@ -343,12 +343,13 @@ struct StreamPlan {
 };
 
 bool slices_legal(int K, int c) { return c >= 2 && K % (c * ck::STREAM_K_MULTIPLE_HOST) == 0 && K / c >= SPLIT_K_MIN_SLICE; }
-// The slices are added inside the kernel where that is allowed - the option; the waves that hold the slices of a wave tile
-// wait for one another, so all of them must be running at once: every workgroup at most one sliced item (sliced_items <=
-// num_cus) and no more workgroups than the device has CUs - and estimated cheaper than the reduction pass.
-bool reduces_in_kernel(const Options& opt, int slices, int64_t sliced_tiles, int64_t mn, int num_cus, int tile_n, int dev_cus) {
-    if (!opt[OPT_FUSED_REDUCTION] || slices < 2 || num_cus > dev_cus || sliced_tiles * slices > num_cus) return false;
-    return opt[OPT_FUSED_REDUCTION] == 2 || fused_reduction_us(slices, tile_n) < reduction_pass_us(slices, mn);
+// The slices are added inside the kernel where the option allows it and that is estimated cheaper than the reduction
+// pass. (No wave waits for another there, so nothing has to be resident together: any number of sliced items per
+// workgroup, any grid.)
+bool reduces_in_kernel(const Options& opt, int slices, int64_t sliced_tiles, int64_t mn, int num_cus) {
+    if (!opt[OPT_FUSED_REDUCTION] || slices < 2) return false;
+    const double per_workgroup = std::ceil((double)sliced_tiles * slices / num_cus);
+    return opt[OPT_FUSED_REDUCTION] == 2 || fused_reduction_us(slices, per_workgroup) < reduction_pass_us(slices, mn);
 }
 
 // Number of K slices for `tiles` tiles that all are cut (1: no split). policy 0: never; 1: automatic - with fewer tiles
@@ -368,7 +369,7 @@ int split_k_slices(int64_t tiles, int64_t mn, int K, int num_cus, const Options&
     double best_us = split_k_estimate_us(tiles, mn, K, 1, num_cus, tile_n, false, dev_cus);
     for (int c = 2; c <= 16; ++c) {
         if (!slices_legal(K, c)) continue;
-        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus, tile_n, reduces_in_kernel(opt, c, tiles, mn, num_cus, tile_n, dev_cus), dev_cus);
+        const double us = split_k_estimate_us(tiles, mn, K, c, num_cus, tile_n, reduces_in_kernel(opt, c, tiles, mn, num_cus), dev_cus);
         if (us < 0.97 * best_us) { best = c; best_us = us; }
     }
     return best;
@@ -404,7 +405,7 @@ StreamPlan stream_plan(int M, int N, int K, int num_cus, const Options& opt) {
         StreamPlan p{tile_n, tiles, tiles, 1, false, persistent_grid(tiles, num_cus, opt[OPT_NUM_XCD], even), 0.0};
         if (tiles <= num_cus) {
             p.slices = split_k_slices(tiles, mn, K, num_cus, opt, tile_n, dev_cus);
-            p.fused = reduces_in_kernel(opt, p.slices, tiles, mn, num_cus, tile_n, dev_cus);
+            p.fused = reduces_in_kernel(opt, p.slices, tiles, mn, num_cus);
             if (p.slices > 1) {
                 p.whole_tiles = 0;
                 p.grid = (int)std::min<int64_t>(tiles * p.slices, num_cus);
@@ -416,7 +417,7 @@ StreamPlan stream_plan(int M, int N, int K, int num_cus, const Options& opt) {
         const double rounds = std::ceil((double)tiles / num_cus), bodies = (double)K / ck::STREAM_K_MULTIPLE_HOST;
         p.us = rounds * round_us_for(even ? (double)tiles / rounds : (double)num_cus, bodies, tile_n, dev_cus);
         const int64_t full = tiles / num_cus * num_cus, rest = tiles - full;
-        if (rest > 0 && opt[OPT_TAIL_ROUND] && opt[OPT_FUSED_REDUCTION] && opt[OPT_SPLIT_K] == 1 && num_cus <= dev_cus) {
+        if (rest > 0 && opt[OPT_TAIL_ROUND] && opt[OPT_FUSED_REDUCTION] && opt[OPT_SPLIT_K] == 1) {
             const double head_us = (double)(full / num_cus) * round_us_for(num_cus, bodies, tile_n, dev_cus);
             for (int c = 2; c <= TAIL_ROUND_MAX_SLICES; ++c) {
                 if (!slices_legal(K, c) || rest * c > num_cus) continue;
@@ -442,13 +443,13 @@ StreamPlan stream_plan(int M, int N, int K, int num_cus, const Options& opt) {
     return best;
 }
 
-// Scratch memory of the K slices of a plan. Reduced in the kernel: per sliced tile slices - 1 tiles of fp32 in the
-// accumulators' layout (what the slices' waves store of the rows they do not own), behind the announcement counters (one
-// 128-byte line per sliced tile and wave, cleared by every launch). Reduced by the second pass: slices planes of M x N fp32.
+// Scratch memory of the K slices of a plan. Reduced in the kernel: per sliced tile `slices` tiles of fp32 in the
+// accumulators' layout (every slice's wave stores its partial sums), behind the arrival counters (one 128-byte line per
+// sliced tile and wave, cleared by every launch). Reduced by the second pass: slices planes of M x N fp32.
 constexpr size_t FIX_STATE_BYTES_PER_TILE = 8 * 128;   // eight waves, one counter per 128-byte line (FIX_STATE_STRIDE_BYTES of the kernel)
 size_t fix_state_bytes(const StreamPlan& p) { return (size_t)(p.tiles - p.whole_tiles) * FIX_STATE_BYTES_PER_TILE; }
 size_t fix_partial_bytes(const StreamPlan& p) {
-    return (size_t)(p.tiles - p.whole_tiles) * (size_t)(p.slices - 1) * 256 * p.tile_n * sizeof(float);
+    return (size_t)(p.tiles - p.whole_tiles) * (size_t)p.slices * 256 * p.tile_n * sizeof(float);
 }
 
 // The tuning tuple the straight-line kernel is written for (it also needs K in whole loop bodies of 64).
@@ -609,7 +610,7 @@ int gemm_launch(int dtype, const void* A, const void* Bt, const void* C, void* D
         if (plan.slices == 1) {
             e = launch(a, plan.grid);
         } else if (plan.fused) {
-            // one launch: the whole tiles, then the (tile, slice) items; a wave tile's last slice to arrive adds the others
+            // one launch: the whole tiles, then the (tile, slice) items; of a wave tile's slices the wave that arrives last adds them all
             GemmArgs p = a;
             p.split_k = plan.slices;
             p.whole_tiles = (int)plan.whole_tiles;

@@ -72,11 +72,10 @@ struct GemmArgs {
     int split_chunk;  // consecutive work items that belong to one slice (32 = one XCD round, or all sliced tiles if fewer)
     int whole_tiles;  // straight-line kernel only: tile counts [0, whole_tiles) are work items over all of K; the K-sliced
                       // items follow them in the item list (all tiles when split_k is 1)
-    // Reduction of the K slices inside the kernel (straight-line kernel): of a wave tile's accumulator block rows the
-    // wave of slice s keeps the rows i with i % split_k == s and stores the others to fix_partials; when all split_k
-    // waves have done so, each adds what the others stored for its rows and writes those rows of D. fix_state holds one
-    // word per (sliced tile, wave) that starts at zero: the number of waves that have stored. Null: no reduction in the
-    // kernel.
+    // Reduction of the K slices inside the kernel (straight-line kernel): every slice's wave stores its partial sums of a
+    // wave tile to fix_partials ([sliced tile][wave][slice][block row], 1 KiB per accumulator block) and counts itself in
+    // fix_state, one word per (sliced tile, wave), 128 bytes apart, that starts at zero; the wave that finds itself the
+    // last adds the partials in slice order and writes the wave tile of D. Null: no reduction in the kernel.
     float* fix_partials;
     unsigned int* fix_state;
     uint32_t spin_limit;
@@ -87,7 +86,7 @@ struct GemmArgs {
                            // ticks workgroup 0 spent in the last launch (actual-clock evidence)
 };
 
-enum : unsigned { CK_STATUS_PRODUCER_TIMEOUT = 1u, CK_STATUS_CONSUMER_TIMEOUT = 2u, CK_STATUS_REDUCTION_TIMEOUT = 4u };
+enum : unsigned { CK_STATUS_PRODUCER_TIMEOUT = 1u, CK_STATUS_CONSUMER_TIMEOUT = 2u };
 
 struct f16_tag {};
 struct bf16_tag {};

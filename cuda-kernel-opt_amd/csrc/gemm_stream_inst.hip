@@ -1,4 +1,5 @@
 // Launchers of the straight-line kernel (one instance per element type, schedule, K-tail form and tile width).
+#include <atomic>
 #include "gemm_stream_kernel.hip.h"
 
 namespace ck {
@@ -9,14 +10,14 @@ template <typename DT, bool ODD_ONLY, bool KTAIL, int WTC>
 static hipError_t stream_launch_one(dim3 grid, hipStream_t stream, const GemmArgs& a) {
     auto kern = gemm_stream_kernel<DT, ODD_ONLY, KTAIL, WTC>;
     constexpr int lds_bytes = stream_lds_bytes(2 * WTC * 16);   // (this file holds the 256- and 128-wide instances; gemm_stream_inst_w6.hip the 192-wide ones)
-    static bool opted[64] = {};
+    static std::atomic<bool> opted[64] = {};   // (threads may launch at once; setting the attribute twice is harmless)
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && !opted[dev]) {
+    if (dev < 0 || dev >= 64 || !opted[dev].load(std::memory_order_acquire)) {
         e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES_PER_CU);
         if (e != hipSuccess) return e;
-        opted[dev] = true;
+        if (dev >= 0 && dev < 64) opted[dev].store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, grid, dim3(512), lds_bytes, stream, a);
     return hipGetLastError();

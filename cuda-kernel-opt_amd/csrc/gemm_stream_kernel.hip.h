@@ -364,77 +364,78 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < WTC; ++j) fb[0][j] = *(const CK_LDS u32x4*)(uintptr_t)(b_lane + (uint32_t)(j * 16 * RB));
 
-        // K slices reduced in the kernel. Each wave handles its own wave tile of D, which S waves hold one slice of:
-        // the wave of slice s owns the accumulator block rows i with i % S == s. It stores its other rows to scratch
-        // memory in the accumulators' own layout (1 KiB per store), announces them, waits until all S waves have
-        // announced, adds what the others stored for its rows to its accumulators - its own slice first, then the
-        // others in slice order, a fixed order per element - and runs the ordinary epilogue on its rows only. The S
-        // waves wait for one another, so they must all be running: the host cuts tiles this way only when every
-        // workgroup gets at most one sliced item (its last) and there are no more workgroups than the device has CUs.
+        // K slices reduced in the kernel, without any wave waiting for another. Each wave handles its own wave tile of
+        // D, of which S waves (one per slice, in S workgroups) hold a partial sum. Every one of them stores its partial to
+        // scratch memory in the accumulators' own layout (1 KiB per store) and then counts itself on the wave tile's
+        // counter; the one that finds itself the last adds the partials in slice order - ((p0 + p1) + p2) + ...
+        // whichever wave comes last, so the result does not depend on the order of arrival and equals the reduction
+        // pass's bit for bit - and runs the ordinary epilogue; the others are done with the tile. Nothing spins: the workgroups of a
+        // launch need not be resident together, and other kernels may compete for the device's CUs.
+        // Returns whether this wave is the one that writes the wave tile to D.
         auto reduce_slices = [&](int64_t tc, int slice) __attribute__((always_inline)) {
-            unsigned own_rows = 0;
-            // The stored rows cross from one XCD's CU to another's, and the L2s of different XCDs do not see each
-            // other's lines. Fences would make that safe by writing back and invalidating whole L2s, once per
-            // wave (measured: 45 us per launch); instead the rows are stored and loaded with system-scope
-            // accesses (sc0 sc1: written through to memory, read past both caches), the announcement follows the
-            // completion of the stores, and no cache is touched as a whole.
+            // The partials cross from one XCD's CU to another's, and the L2s of different XCDs do not see each other's
+            // lines. Fences would make that safe by writing back and invalidating whole L2s, once per wave (measured:
+            // 45 us per launch); instead the partials are stored and loaded with system-scope accesses (sc0 sc1:
+            // written through to memory, read past both caches), a wave counts itself only after its stores have
+            // completed, and no cache is touched as a whole.
             constexpr int ROW_BYTES = WTC * 1024;          // one block row of a wave tile: 16 bytes per lane and block
             constexpr int SYSTEM_SCOPE = 1 | 16;           // sc0 | sc1 of a buffer access
             const int unit = __builtin_amdgcn_readfirstlane((int)(tc - T1) * 8 + wave);
-            // (one counter per 128-byte line: thousands of waves poll them, and counters that share a line share a memory channel)
-            unsigned int* announced = g.fix_state + (size_t)unit * (FIX_STATE_STRIDE_BYTES / 4);
-            // per (tile, wave): [block row][contributor: the S - 1 slices that do not own the row, in slice order]
-            const int unit_bytes = WTR * (S - 1) * ROW_BYTES;
+            // (one counter per 128-byte line: counters that share a line share a memory channel)
+            unsigned int* arrived = g.fix_state + (size_t)unit * (FIX_STATE_STRIDE_BYTES / 4);
+            // per (tile, wave): [slice][block row]
+            const int unit_bytes = S * WTR * ROW_BYTES;
             const __amdgpu_buffer_rsrc_t rows = __builtin_amdgcn_make_buffer_rsrc((char*)g.fix_partials + (size_t)unit * (size_t)unit_bytes, 0,
                                                                                   unit_bytes, 0x00020000);
             const int ln16 = lane * 16;
-            own_rows = 0;
+            const int mine = __builtin_amdgcn_readfirstlane(slice * WTR * ROW_BYTES);
 #pragma unroll
-            for (int i = 0; i < WTR; ++i) {
-                const int owner = i % S;
-                if (owner == slice) {
-                    own_rows |= 1u << i;
-                } else {
-                    const int at = __builtin_amdgcn_readfirstlane((i * (S - 1) + (slice < owner ? slice : slice - 1)) * ROW_BYTES);
+            for (int i = 0; i < WTR; ++i)
 #pragma unroll
-                    for (int j = 0; j < WTC; ++j)
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rows, ln16, at + j * 1024, SYSTEM_SCOPE);
-                }
-            }
-            own_rows = __builtin_amdgcn_readfirstlane(own_rows);
-            // the stores are complete (in memory) before the announcement
+                for (int j = 0; j < WTC; ++j)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rows, ln16, mine + i * ROW_BYTES + j * 1024, SYSTEM_SCOPE);
+            // the stores are complete (in memory) before the wave counts itself
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            if (lane == 0) __hip_atomic_fetch_add(announced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            for (uint32_t n = 0;; ++n) {
-                const uint32_t seen = __builtin_amdgcn_readfirstlane(__hip_atomic_load(announced, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-                if ((int)seen >= S) break;
-                if (n > g.spin_limit) {   // the grid drains whatever happens; the status word says D is invalid
-                    if (lane == 0) atomicOr(g.status, CK_STATUS_REDUCTION_TIMEOUT);
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(8);
-            }
+            unsigned int before = 0;
+            if (lane == 0) before = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            before = __builtin_amdgcn_readfirstlane(before);
             asm volatile("" ::: "memory");
+            if ((int)before != S - 1) return false;   // another wave will come last
+            // Slice order without a second set of accumulators: p0 + p1 is p1 + p0, so the wave of slice 0 or 1 starts
+            // from its registers and adds the other of the two; a wave of a later slice starts from p0 and takes its own
+            // partial from memory like the others, in its place. Then p2, p3, ... (A partial sum starts from +0 and is
+            // never -0, so starting from the first partial and starting from 0 + the first partial are the same.)
+            const bool from_registers = slice <= 1;
+            const int first = from_registers ? 1 - slice : 0, next = from_registers ? 2 : 1;
 #pragma unroll
             for (int i = 0; i < WTR; ++i) {
-                if (own_rows & (1u << i)) {
-                    // one contributor after the other, in slice order (deeper queues - two or three contributors' loads in
-                    // flight - measured no faster: what this phase costs is the wait for the slowest slice, not the loads)
-                    for (int c = 0; c < S - 1; ++c) {
-                        const int at = __builtin_amdgcn_readfirstlane((i * (S - 1) + c) * ROW_BYTES);
-                        u32x4 x[WTC];
+                {
+                    const int at = __builtin_amdgcn_readfirstlane((first * WTR + i) * ROW_BYTES);
+                    u32x4 x[WTC];
 #pragma unroll
-                        for (int j = 0; j < WTC; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b128(rows, ln16, at + j * 1024, SYSTEM_SCOPE);
+                    for (int j = 0; j < WTC; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b128(rows, ln16, at + j * 1024, SYSTEM_SCOPE);
 #pragma unroll
-                        for (int j = 0; j < WTC; ++j) acc[i][j] += __builtin_bit_cast(f32x4, x[j]);
+                    for (int j = 0; j < WTC; ++j) {
+                        f32x4 start;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) start[e] = from_registers ? acc[i][j][e] : 0.f;
+                        acc[i][j] = start + __builtin_bit_cast(f32x4, x[j]);
                     }
                 }
+                for (int c = next; c < S; ++c) {
+                    const int at = __builtin_amdgcn_readfirstlane((c * WTR + i) * ROW_BYTES);
+                    u32x4 x[WTC];
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b128(rows, ln16, at + j * 1024, SYSTEM_SCOPE);
+#pragma unroll
+                    for (int j = 0; j < WTC; ++j) acc[i][j] += __builtin_bit_cast(f32x4, x[j]);
+                }
             }
-            return own_rows;
+            return true;
         };
-        // D = alpha * acc + beta * C for the block rows `own_rows` of this wave's wave tile, straight from the accumulators;
+        // D = alpha * acc + beta * C for this wave's wave tile, straight from the accumulators;
         // returns whether the tile is an interior one (every wave then issues exactly the stores the next body's landing wait counts)
-        auto write_tile = [&](int64_t tc, int slice, unsigned own_rows) __attribute__((always_inline)) {
+        auto write_tile = [&](int64_t tc, int slice) __attribute__((always_inline)) {
             // Every value of C fetched ahead of its use passes through here at the point of use, on every path. The
             // compiler waits for a load where its result is used; when it moves the use under a condition (a row past the
             // edge, beta == 0), the paths that skip the use leave the load in flight as far as it can tell, all the way
@@ -495,7 +496,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                             for (int tt = 0; tt < STORES_PER_GROUP; ++tt) {
                                 const f32x4 v = exchanged(i, j, tt);
                                 const int64_t row = row0 + i * 16 + tt * 8;
-                                if (row < g.M && (own_rows & (1u << i))) put(row * g.N + (col0 + j * 16), v);
+                                if (row < g.M) put(row * g.N + (col0 + j * 16), v);
                             }
                         }
                     }
@@ -504,10 +505,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                     // by one between the stores (a load may not pass the store in front of it)
                     constexpr int C_DEPTH = 4;
                     f32x4 cv[C_DEPTH];
-                    auto row_of = [&](int st) {   // (a block row another slice's wave writes counts as past the edge)
-                        return (own_rows & (1u << (st / (GROUPS * STORES_PER_GROUP)))) ? row0 + (st / (GROUPS * STORES_PER_GROUP)) * 16 + (st % STORES_PER_GROUP) * 8
-                                                                                     : (int64_t)g.M;
-                    };
+                    auto row_of = [&](int st) { return row0 + (st / (GROUPS * STORES_PER_GROUP)) * 16 + (st % STORES_PER_GROUP) * 8; };
                     auto off_of = [&](int st) { return row_of(st) * g.N + (col0 + ((st / STORES_PER_GROUP) % GROUPS) * F32_GROUP * 16); };
                     auto fetch = [&](int st) __attribute__((always_inline)) {
                         return row_of(st) < g.M ? (f32x4)*(const f32x4_u*)(go.C + off_of(st)) : f32x4{0.f, 0.f, 0.f, 0.f};
@@ -578,7 +576,6 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                         const int gi = i * GROUPS16 + j / H16_GROUP;   // this group; the next one's C goes into the other buffer
                         if (gi + 1 < WTR * GROUPS16) fetch_c((gi + 1) / GROUPS16, ((gi + 1) % GROUPS16) * H16_GROUP, cq[(gi + 1) % 2]);
                         landed(cq[gi % 2][0]); landed(cq[gi % 2][1]); landed(cq[gi % 2][2]); landed(cq[gi % 2][3]);
-                        if (!(own_rows & (1u << i))) continue;   // a block row another slice's wave writes
                         const u32x4 first = packed_pair(scaled(acc[i][j], cq[gi % 2][0]), scaled(acc[i][j + 1], cq[gi % 2][1]));
                         const u32x4 second = packed_pair(scaled(acc[i][j + 2], cq[gi % 2][2]), scaled(acc[i][j + 3], cq[gi % 2][3]));
                         u32x4 other;  // the second pair's piece of the row 8 away
@@ -603,7 +600,7 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                 for (int i = 0; i < WTR; ++i)
 #pragma unroll
                     for (int j = 0; j < WTC; ++j)
-                        if (own_rows & (1u << i)) epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], vec_cols);
+                        epilogue_block<DT>(go, m_base + i * 16, n_base + j * 16, acc[i][j], vec_cols);
             }
             return interior;
         };
@@ -625,12 +622,14 @@ __global__ __launch_bounds__(512) void gemm_stream_kernel(const GemmArgs g) {
                     q0 = n0; q1 = n1; q2 = n2; q4 = n4;
                 }
             }
-            unsigned own_rows = (1u << WTR) - 1;   // block rows of the wave tile this wave writes to D
+            // a sliced tile whose slices are added in the kernel is written by the wave that comes last
             const bool reduce_here = !KTAIL && sliced && g.fix_partials != nullptr;
+            bool writes = true;
             if constexpr (!KTAIL) {
-                if (reduce_here) own_rows = reduce_slices(tc, slice);
+                if (reduce_here) writes = reduce_slices(tc, slice);
             }
-            const bool interior = write_tile(tc, slice, own_rows) && !reduce_here;
+            bool interior = false;
+            if (writes) interior = write_tile(tc, slice) && !reduce_here;
 #pragma unroll
             for (int i = 0; i < WTR; ++i)
 #pragma unroll

@@ -1,4 +1,5 @@
 // Launchers of the synchronous single-stage kernel (the no-pipeline, no-specialisation A/B partner).
+#include <atomic>
 #include "gemm_sync_kernel.hip.h"
 
 namespace ck {
@@ -6,14 +7,14 @@ namespace ck {
 template <typename DT, int TILE, int SEGK, int CW>
 static hipError_t sync_launch_one(dim3 grid, size_t lds, hipStream_t stream, const GemmArgs& a) {
     auto kern = gemm_sync_kernel<DT, TILE, SEGK, CW>;
-    static bool opted[64] = {};
+    static std::atomic<bool> opted[64] = {};   // (threads may launch at once; setting the attribute twice is harmless)
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && !opted[dev]) {
+    if (dev < 0 || dev >= 64 || !opted[dev].load(std::memory_order_acquire)) {
         e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES_PER_CU);
         if (e != hipSuccess) return e;
-        opted[dev] = true;
+        if (dev >= 0 && dev < 64) opted[dev].store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, grid, dim3(CW * WAVE), lds, stream, a);
     return hipGetLastError();

@@ -300,15 +300,16 @@ int ckopt_last_launch_clocks(void* stream, uint64_t* shader_cycles, uint64_t* re
  * key 12: the partly filled last round of the straight-line kernel (default 1). With more tiles than num_sms the last
  *        round leaves CUs idle (6144^3: 576 tiles = 2 x 256 + 64); with 1 its tiles are cut into 2 to 4 K slices that
  *        run as work items of the same launch behind the whole tiles, where the cost model gives that at least 3 % less
- *        time than evenly filled rounds of whole tiles (key 9); needs keys 7 and 13 at 1. 0: never.
- * key 13: where K slices are added. Inside the straight-line kernel: of every wave tile each slice's wave keeps some of
- *        the accumulator block rows, stores the others to scratch memory ((slices - 1) x tile bytes and 1 KiB of counters
- *        per cut tile), waits for the other slices' waves and adds what they stored for its rows, in a fixed order per
- *        element (deterministic), and writes those rows of D; no second kernel. It needs every workgroup to hold at most
- *        one sliced item (tiles x slices <= num_sms) and no more workgroups than the device has CUs. Or by a second
- *        kernel over slices x M x N x 4 bytes of planes. 1 (default): inside the kernel where that is possible and the
- *        cost model gives it less time (two slices of a large product: 18 us against 22; four slices of 2048 x 2048:
- *        42 against 19, most of it the wait for the slowest slice); 2: wherever possible; 0: never.
+ *        time than evenly filled rounds of whole tiles (key 9); needs key 7 at 1 and key 13 not 0. 0: never.
+ * key 13: where K slices are added. Inside the straight-line kernel: every slice's wave stores its partial sums of a
+ *        wave tile to scratch memory (slices x tile bytes and 1 KiB of counters per cut tile) and counts itself on the
+ *        wave tile's counter; the wave that finds itself the last adds the partials in slice order - the same order
+ *        whichever comes last, so the result is deterministic and equal to the second kernel's bit for bit - and writes
+ *        D; no second kernel, and no wave waits for another (launches may overlap with anything). Or by a second
+ *        kernel over slices x M x N x 4 bytes of planes. 1 (default): inside the kernel where the cost model gives it
+ *        less time (measured: two slices of 128 tiles 27 us against 22 for the second kernel, four of 64 tiles 47
+ *        against 19 - the last wave's chain of memory round trips - so on a 256-CU device the second kernel is what
+ *        runs); 2: always inside the kernel; 0: never.
  * key 14: wave-tile granularity of the counter-synchronised kernel (default 1). 1: a producer wave reads all "released"
  *        counters of its operand and stage in one look per segment and polls a row block's counter only if that look
  *        found it short; 0: it polls every row block's counter on its own, as the reference's producers wait on every

@@ -825,18 +825,20 @@ def test_split_k_bit_exact(ck, M, N, K, slices, cus, dt_name):
 
 @pytest.mark.parametrize("M,N,K,cus,opts", [
     (2048, 4096, 4096, 256, dict(split_k=2)),            # 128 tiles, two slices: every workgroup one item
-    (512, 512, 8192, 256, dict(split_k=4)),              # 4 tiles x 4 slices: a wave owns one block row
-    (700, 520, 6144, 256, dict(split_k=3)),              # ragged tiles, three slices: slice 0 owns two block rows
-    (512, 768, 16384, 256, dict(split_k=16)),            # 6 tiles x 16 slices: slices 4 .. 15 own nothing
+    (512, 512, 8192, 256, dict(split_k=4)),              # 4 tiles x 4 slices
+    (700, 520, 6144, 256, dict(split_k=3)),              # ragged tiles, three slices
+    (512, 768, 16384, 256, dict(split_k=16)),            # 6 tiles x 16 slices
     (1024, 1280, 8192, 16, dict()),                      # the partly filled last round: 16 whole tiles + 4 sliced, one launch
-    (2048, 1280, 4096, 16, dict()),                      # two full rounds + 8 sliced tiles
+    (2048, 1280, 8192, 16, dict()),                      # two full rounds + 8 sliced tiles
     (1000, 640, 8192, 8, dict(half_width=2)),            # 256 x 128 tiles: 4 x 5 on 8 workgroups, ragged in M
     (1400, 1200, 4096, 8, dict(tail_round=0)),
+    (512, 768, 8192, 6, dict(split_k=4)),                # 6 tiles x 4 slices on 6 workgroups: four sliced items each, one after the other
+    (512, 500, 6144, 6, dict(split_k=3, half_width=3)),  # 256 x 192 tiles: 2 x 3 tiles x 3 slices on 6 workgroups, ragged in N
 ])
 def test_slices_reduced_in_the_kernel_exact(ck, M, N, K, cus, opts):
-    """K slices added inside the straight-line kernel (no second kernel): fp32 and 16-bit output, with and without C, exact
-    on small integers; the same bits as the two-kernel form on random data (both add the slices of an element in a fixed
-    order, but not the same one, so the comparison there is within rounding of the sums)."""
+    """K slices added inside the straight-line kernel (no second kernel; of a wave tile's slices the wave that arrives last
+    adds them all, in slice order, and writes D): fp32 and 16-bit output, with and without C, exact on small integers, any
+    number of sliced items per workgroup."""
     t = _straight_line_tuning(ck, cus)
     tup = tuple(t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
                                "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms"))
@@ -874,10 +876,10 @@ def test_slices_reduced_in_the_kernel_exact(ck, M, N, K, cus, opts):
         assert e.value.code == ck.ERR_TOO_LARGE
 
 
-def test_slices_reduced_in_the_kernel_against_the_second_pass(ck, oracle):
-    """Random fp16 data, 128 tiles in two slices: the two forms of the reduction agree to the last bits of an fp32 sum of two
-    terms in different order (they are equal: two terms have one order), and both are within tolerance of the oracle."""
-    M, N, K = 2048, 4096, 4096
+@pytest.mark.parametrize("M,N,K,slices", [(2048, 4096, 4096, 2), (2048, 2048, 8192, 4), (1024, 768, 6144, 3)])
+def test_slices_reduced_in_the_kernel_against_the_second_pass(ck, oracle, M, N, K, slices):
+    """Random fp16 data: both forms of the reduction add the slices of an element in slice order - in the kernel
+    whichever wave arrives last - so they agree bit for bit, run after run; and both are within tolerance of the oracle."""
     t = _straight_line_tuning(ck, 256)
     tup = tuple(t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
                                "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms"))
@@ -885,16 +887,46 @@ def test_slices_reduced_in_the_kernel_against_the_second_pass(ck, oracle):
     bt = ck.fill_uniform(ck.DT_F16, (N, K), 99, 1, -1.0, 1.0)
     da, db = G.to_dev(a), G.to_dev(bt)
     out = []
-    for fused in (2, 0):
-        o = ck.launch_options(split_k=2, fused_reduction=fused)
-        assert ck.gemm_launch_plan(M, N, K, True, *tup, options=o)["reduced_in_kernel"] == bool(fused)
+    for fused in (2, 0, 2):
+        o = ck.launch_options(split_k=slices, fused_reduction=fused, half_width=0)
+        plan = ck.gemm_launch_plan(M, N, K, True, *tup, options=o)
+        assert plan["reduced_in_kernel"] == bool(fused) and plan["k_slices"] == slices, plan
         d = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
         ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, da, db, None, d, 1.0, 0.0, M, N, K, *tup, options=o)
         assert ck.device_status() == 0
         out.append(d.cpu().numpy())
-    assert np.array_equal(out[0], out[1])
+    assert np.array_equal(out[0], out[1]) and np.array_equal(out[0], out[2])
     ref = oracle.gemm(oracle.DT_F16, a, bt, rows=(0, 256))
     assert_close(oracle, ref, out[0][:256])
+
+
+def test_two_streams_reduce_in_the_kernel_at_once(ck):
+    """Launches that add their K slices inside the kernel, issued on two streams at the same time: each needs the whole
+    device (256 work items), so their workgroups compete for the CUs and neither launch is resident as a whole. No wave
+    waits for another in that reduction, so both finish and both are exact."""
+    M, N, K = 2048, 2048, 8192
+    t = _straight_line_tuning(ck, 256)
+    tup = tuple(t[k] for k in ("tile_dim", "segment_dim_k", "bar_steps_a", "bar_steps_b", "bar_step_rows_a", "bar_step_rows_b", "tile_group_m",
+                               "num_stages", "num_producer_warps", "num_consumer_warps", "num_sms"))
+    o = ck.launch_options(split_k=4, fused_reduction=2, half_width=0)
+    assert ck.gemm_launch_plan(M, N, K, True, *tup, options=o)["reduced_in_kernel"]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    ops, wants, outs = [], [], []
+    for i in range(2):
+        a = ck.fill_int(ck.DT_F16, (M, K), 300 + i, 0, -2, 2)
+        bt = ck.fill_int(ck.DT_F16, (N, K), 300 + i, 1, -2, 2)
+        wants.append((a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32))
+        ops.append((G.to_dev(a), G.to_dev(bt)))
+        outs.append(torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda"))
+    torch.cuda.synchronize()
+    for rep_ in range(6):
+        for i in range(2):
+            ck.gemm_shmem_tc_async_opt_port_ex(ck.DT_F16, ck.DT_F32, ops[i][0], ops[i][1], None, outs[i], 1.0, 0.0, M, N, K, *tup, options=o,
+                                               stream=streams[i])
+    torch.cuda.synchronize()
+    assert ck.device_status() == 0
+    for i in range(2):
+        assert np.array_equal(outs[i].cpu().numpy(), wants[i]), i
 
 
 def test_two_host_threads_with_different_options(ck):
@@ -1095,8 +1127,8 @@ def test_automatic_split_k_of_128_tiles_exact(ck):
     for width, planes in ((0, 2), (1, 0)):
         prev = ck.set_option(ck.OPT_HALF_WIDTH, width)
         try:
-            # (two slices of this size are added inside the kernel: one tile of fp32 and eight counter lines per tile)
-            assert ck.gemm_workspace_bytes(M, N, K, True, *order) == (128 * (256 * 256 * 4 + 8 * 128) + 256 if planes else 0)
+            # (the two slices are added by the second pass: two planes of M x N fp32)
+            assert ck.gemm_workspace_bytes(M, N, K, True, *order) == (planes * M * N * 4 + 256 if planes else 0)
             assert ck.gemm_launch_plan(M, N, K, True, *order)["k_slices"] == (planes if planes else 1)
             assert np.array_equal(G.run_gemm(ck, ck.DT_F16, a, bt, t=t), want), width
         finally:

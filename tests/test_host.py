@@ -384,11 +384,13 @@ def test_workspace_query_follows_the_launcher_rules(ck):
     assert ck.gemm_workspace_bytes(1536, 1536, 8192, True, *straight) == 4 * 1536 * 1536 * 4 + 256
     # the automatic slice count follows the launcher's cost model: 128 tiles with a deep K are cut in two (256 items),
     # with K 4096 not at all (the reduction pass would cost more than the idle half of the CUs); 81 tiles in three;
-    # 144 tiles never (two slices would be 288 items: two rounds). Two slices of a large product are added inside the
-    # kernel: per tile one tile of fp32 (what each slice's waves store of the rows they do not own) and eight 128-byte
-    # counter lines, instead of two M x N planes
-    assert ck.gemm_workspace_bytes(2048, 4096, 16384, True, *straight) == 128 * 8 * 128 + 128 * 256 * 256 * 4 + 256
+    # 144 tiles never (two slices would be 288 items: two rounds). The slices are added by the second pass (planes of
+    # M x N fp32) unless the option asks for the reduction inside the kernel: then per tile and slice one tile of fp32
+    # (every slice's waves store their partial sums) behind eight 128-byte counter lines per tile
+    assert ck.gemm_workspace_bytes(2048, 4096, 16384, True, *straight) == 2 * 2048 * 4096 * 4 + 256
     assert ck.gemm_workspace_bytes(2048, 4096, 16384, True, *straight, options=ck.launch_options(fused_reduction=0)) == 2 * 2048 * 4096 * 4 + 256
+    assert (ck.gemm_workspace_bytes(2048, 4096, 16384, True, *straight, options=ck.launch_options(fused_reduction=2))
+            == 128 * 8 * 128 + 2 * 128 * 256 * 256 * 4 + 256)
     assert ck.gemm_workspace_bytes(2048, 4096, 4096, True, *straight) == 0
     assert ck.gemm_workspace_bytes(2304, 2304, 12288, True, *straight) == 3 * 2304 * 2304 * 4 + 256
     assert ck.gemm_workspace_bytes(3072, 3072, 8192, True, *straight) == 0
@@ -414,7 +416,8 @@ def test_launch_plan_reports_what_a_launch_will_run(ck):
     assert plan(2048, 2048, 32768, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=4, operand_copies=False, sliced_tiles=64,
                                                             reduced_in_kernel=False, grid=256)
     assert plan(2048, 4096, 16384, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=2, operand_copies=False, sliced_tiles=128,
-                                                            reduced_in_kernel=True, grid=256)
+                                                            reduced_in_kernel=False, grid=256)
+    assert plan(2048, 4096, 16384, True, *straight, options=ck.launch_options(fused_reduction=2))["reduced_in_kernel"]
     assert plan(6143, 4097, 3071, True, *straight) == dict(straight_line=True, tile_cols=256, k_slices=1, operand_copies=True, sliced_tiles=0,
                                                            reduced_in_kernel=False, grid=208)
     assert plan(2560, 2560, 2560, True, *straight) == dict(straight_line=True, tile_cols=128, k_slices=1, operand_copies=False, sliced_tiles=0,
