@@ -8,6 +8,8 @@ full-size runs checked through sampled rows and size-independent identities.
 """
 import itertools
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -1370,10 +1372,12 @@ def test_workspace_query_and_launches_that_need_none(ck):
 def test_random_tunings_entry_points_and_options_exact(ck):
     # seeded sweep over every kernel design, synchronisation granularity, grid size, the process-wide options and the
     # three homes of the scratch memory (stream-ordered allocation, caller's workspace, the library's static array):
-    # exact on small integers whatever the summation order; D starts out as NaN, so every element must be written
-    rng = np.random.default_rng(20251126)
+    # exact on small integers whatever the summation order; D starts out as NaN, so every element must be written.
+    # CKOPT_SWEEP_SEED / CKOPT_SWEEP_CASES run the same sweep from another seed or for longer.
+    seed, cases = int(os.environ.get("CKOPT_SWEEP_SEED", "20251126")), int(os.environ.get("CKOPT_SWEEP_CASES", "260"))
+    rng = np.random.default_rng(seed)
     ran = 0
-    for case in range(260):
+    for case in range(cases):
         if rng.random() < 0.35:
             t = G.tuning(tile_dim=256, segment_dim_k=32, num_stages=5, num_producer_warps=0, num_consumer_warps=8,
                          tile_group_m=int(rng.integers(1, 7)), num_sms=int(rng.choice([1, 3, 8, 40, 256])))
@@ -1401,7 +1405,8 @@ def test_random_tunings_entry_points_and_options_exact(ck):
         alpha, beta = float(rng.choice([1.0, 2.0, -0.5])), float(rng.choice([0.0, 0.0, -1.0, 2.0]))
         opts = {ck.OPT_SPLIT_K: int(rng.choice([0, 1, 1, 2, 3, 4, 8])), ck.OPT_BARRIER_EVERY_KSTEP: int(rng.integers(0, 2)),
                 ck.OPT_EVEN_ROUNDS: int(rng.integers(0, 2)), ck.OPT_TILE_SYNC_BARRIER: int(rng.integers(0, 2)),
-                ck.OPT_HALF_WIDTH: int(rng.integers(0, 3)), ck.OPT_D_STORE_POLICY: int(rng.integers(0, 3))}
+                ck.OPT_HALF_WIDTH: int(rng.integers(0, 4)), ck.OPT_D_STORE_POLICY: int(rng.integers(0, 3)),
+                ck.OPT_FUSED_REDUCTION: int(rng.integers(0, 3)), ck.OPT_TAIL_ROUND: int(rng.integers(0, 2))}
         entry = int(rng.integers(0, 3))
         if ck.check_gemm_tuning(*order) != ck.OK:
             continue
@@ -1435,4 +1440,4 @@ def test_random_tunings_entry_points_and_options_exact(ck):
         finally:
             for k, v in prev.items():
                 ck.set_option(k, v)
-    assert ran >= 150
+    assert ran >= 0.55 * cases
